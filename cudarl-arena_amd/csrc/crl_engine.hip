@@ -1,0 +1,792 @@
+// C ABI of the engine (include/crl.h): owns the device buffers, validates
+// arguments on the host and launches the gfx950 kernels of crl_kernels.h.
+// There is no CPU fallback anywhere in this file.
+#include <hip/hip_runtime.h>
+
+#include <cstdarg>
+#include <cstdio>
+#include <cstring>
+#include <new>
+#include <string>
+#include <vector>
+
+#include "../../include/crl.h"
+#include "crl_host.h"
+#include "crl_kernels.h"
+
+namespace {
+
+thread_local std::string g_err;
+
+int fail(int code, const char* fmt, ...) {
+  char buf[512];
+  va_list ap;
+  va_start(ap, fmt);
+  vsnprintf(buf, sizeof buf, fmt, ap);
+  va_end(ap);
+  g_err = buf;
+  return code;
+}
+
+#define HIP_TRY(expr)                                                                   \
+  do {                                                                                  \
+    hipError_t _e = (expr);                                                             \
+    if (_e != hipSuccess)                                                               \
+      return fail(_e == hipErrorOutOfMemory ? CRL_E_ALLOC : CRL_E_DEVICE, "%s: %s (%s:%d)", \
+                  #expr, hipGetErrorString(_e), __FILE__, __LINE__);                    \
+  } while (0)
+
+template <class T>
+struct DevBuf {
+  T* p = nullptr;
+  size_t n = 0;
+  hipError_t alloc(size_t count) {
+    release();
+    if (count == 0) return hipSuccess;
+    hipError_t e = hipMalloc(reinterpret_cast<void**>(&p), count * sizeof(T));
+    if (e == hipSuccess) n = count;
+    else p = nullptr;
+    return e;
+  }
+  hipError_t ensure(size_t count) { return count <= n ? hipSuccess : alloc(count); }
+  void release() {
+    if (p) (void)hipFree(p);
+    p = nullptr;
+    n = 0;
+  }
+  ~DevBuf() { release(); }
+  DevBuf() = default;
+  DevBuf(const DevBuf&) = delete;
+  DevBuf& operator=(const DevBuf&) = delete;
+};
+
+}  // namespace
+
+struct crl_engine {
+  crl_config cfg{};
+  int device = 0;
+  hipStream_t stream = nullptr;
+  int N = 0, W = 0, H = 0, A = 0;
+  size_t S = 0, K = 0;
+  int n_maps = 0, n_tables = 0, map_words = 0;
+  uint64_t t = 0;
+
+  DevBuf<int32_t> s, ep_step, episode, start, act;
+  DevBuf<float> reward;
+  DevBuf<uint8_t> done, action;
+  DevBuf<uint32_t> map;
+  DevBuf<float> cell_reward;
+  DevBuf<float> Q;
+  DevBuf<float> eps_tab;
+  int eps_len = 1;
+  // transition of the last crl_step
+  DevBuf<int32_t> tr_s, tr_a, tr_s2;
+  DevBuf<float> tr_r;
+  DevBuf<uint8_t> tr_done;
+  bool have_transition = false, have_actions = false;
+  // (key, delta) scratch of the ordered reduction
+  DevBuf<int32_t> key;
+  DevBuf<float> delta;
+  // scratch of crl_td_update
+  DevBuf<int32_t> b_s, b_a, b_s2;
+  DevBuf<float> b_r;
+  DevBuf<uint8_t> b_done;
+  // trace
+  DevBuf<int32_t> trace_s;
+  DevBuf<uint8_t> trace_a, trace_d;
+  DevBuf<float> trace_r;
+  int trace_n = 0, trace_cap = 0, trace_cursor = 0;
+  // supplied exploration stream
+  DevBuf<float> u_sup;
+  DevBuf<int32_t> a_sup;
+  uint64_t sup_t0 = 0;
+  int sup_n = 0;
+  // host mirrors for crl_set_cell
+  std::vector<uint8_t> h_class;
+  std::vector<float> h_cell_reward;
+
+  crl::Rules rules() const {
+    crl::Rules R{};
+    R.W = W;
+    R.H = H;
+    R.A = A;
+    R.goal_mode = cfg.goal_mode;
+    R.reward_flags = cfg.reward_flags;
+    R.auto_reset = cfg.auto_reset;
+    R.episode_len = cfg.episode_len;
+    R.max_mode = cfg.max_mode;
+    R.eps_mode = cfg.eps_mode;
+    R.eps_len = eps_len;
+    R.lr = cfg.lr;
+    R.gamma = cfg.gamma;
+    R.step_reward = cfg.step_reward;
+    R.goal_reward = cfg.goal_reward;
+    R.trap_reward = cfg.trap_reward;
+    R.eps0 = cfg.eps0;
+    R.seed = cfg.seed;
+    return R;
+  }
+  crl::Ptrs ptrs() const {
+    crl::Ptrs P{};
+    P.s = s.p;
+    P.ep_step = ep_step.p;
+    P.episode = episode.p;
+    P.start = start.p;
+    P.reward = reward.p;
+    P.done = done.p;
+    P.action = action.p;
+    P.map = map.p;
+    P.cell_reward = (cfg.reward_flags & CRL_REWARD_CELLS) ? cell_reward.p : nullptr;
+    P.Q = Q.p;
+    P.eps_tab = eps_tab.p;
+    P.u_sup = sup_n > 0 ? u_sup.p : nullptr;
+    P.a_sup = a_sup.p;
+    P.sup_t0 = sup_t0;
+    P.sup_n = sup_n;
+    P.tr_s = trace_s.p;
+    P.tr_a = trace_a.p;
+    P.tr_r = trace_r.p;
+    P.tr_d = trace_d.p;
+    P.trace_n = trace_n;
+    P.trace_cursor = trace_cursor;
+    P.trace_cap = trace_cap;
+    P.N = N;
+    P.map_words = map_words;
+    P.map_shared = cfg.map_mode == CRL_MAP_SHARED;
+    P.table_shared = cfg.table_mode == CRL_TABLE_SHARED;
+    P.S = S;
+    return P;
+  }
+  crl::Transition transition() const {
+    crl::Transition T{};
+    T.s = tr_s.p;
+    T.a = tr_a.p;
+    T.r = tr_r.p;
+    T.s2 = tr_s2.p;
+    T.done = tr_done.p;
+    return T;
+  }
+};
+
+namespace {
+
+constexpr int kLdsMapLimitBytes = 64 * 1024;
+
+// launch geometry of the fused per-env kernel
+struct FusedPlan {
+  int map_kind;  // 0 per-env LDS, 1 shared LDS, 2 global
+  int block, grid;
+  size_t lds;
+  const char* name;
+};
+
+FusedPlan plan_fused(const crl_engine* e) {
+  FusedPlan p{};
+  // small batches spread over more compute units with one-wave blocks
+  p.block = e->N >= 256 * 512 ? 256 : 64;
+  if (e->cfg.map_mode == CRL_MAP_SHARED) {
+    if ((size_t)e->map_words * 4 <= (size_t)kLdsMapLimitBytes) {
+      p.map_kind = 1;
+      p.lds = (size_t)e->map_words * 4;
+    } else {
+      p.map_kind = 2;
+    }
+  } else {
+    if ((size_t)e->map_words * 4 * 64 <= (size_t)kLdsMapLimitBytes) {
+      p.map_kind = 0;
+      while ((size_t)e->map_words * 4 * p.block > (size_t)kLdsMapLimitBytes) p.block /= 2;
+      p.lds = (size_t)e->map_words * 4 * p.block;
+    } else {
+      p.map_kind = 2;
+    }
+  }
+  p.grid = (e->N + p.block - 1) / p.block;
+  static const char* names[2][3] = {
+      {"k_fused_per_env<4,0>", "k_fused_per_env<4,1>", "k_fused_per_env<4,2>"},
+      {"k_fused_per_env<8,0>", "k_fused_per_env<8,1>", "k_fused_per_env<8,2>"}};
+  p.name = names[e->A == 8][p.map_kind];
+  return p;
+}
+
+template <int A>
+void launch_fused_a(const crl_engine* e, const FusedPlan& p, uint64_t t0, int n) {
+  const crl::Rules R = e->rules();
+  const crl::Ptrs P = e->ptrs();
+  switch (p.map_kind) {
+    case 0:
+      hipLaunchKernelGGL((crl::k_fused_per_env<A, 0>), dim3(p.grid), dim3(p.block), p.lds, e->stream,
+                         R, P, t0, n);
+      break;
+    case 1:
+      hipLaunchKernelGGL((crl::k_fused_per_env<A, 1>), dim3(p.grid), dim3(p.block), p.lds, e->stream,
+                         R, P, t0, n);
+      break;
+    default:
+      hipLaunchKernelGGL((crl::k_fused_per_env<A, 2>), dim3(p.grid), dim3(p.block), 0, e->stream, R, P,
+                         t0, n);
+      break;
+  }
+}
+
+int reduce_apply(crl_engine* e, float* Q, const int32_t* key, const float* delta, int n) {
+  const int grid = (int)((e->K + crl::kOwnKeys - 1) / crl::kOwnKeys);
+  hipLaunchKernelGGL(crl::k_reduce_apply, dim3(grid), dim3(crl::kReduceBlock), 0, e->stream, Q,
+                     (int)e->K, key, delta, n);
+  HIP_TRY(hipGetLastError());
+  return CRL_OK;
+}
+
+// one shared-table step: act (select+move+delta), then ordered reduce + apply
+int shared_step(crl_engine* e, uint64_t t, int trace_row) {
+  const crl::Rules R = e->rules();
+  const crl::Ptrs P = e->ptrs();
+  const int block = 256, grid = (e->N + block - 1) / block;
+  const bool lds_map =
+      e->cfg.map_mode == CRL_MAP_SHARED && (size_t)e->map_words * 4 <= (size_t)kLdsMapLimitBytes;
+  const size_t lds = lds_map ? (size_t)e->map_words * 4 : 0;
+  if (e->A == 4) {
+    if (lds_map)
+      hipLaunchKernelGGL((crl::k_shared_act<4, 1>), dim3(grid), dim3(block), lds, e->stream, R, P, t,
+                         trace_row, e->key.p, e->delta.p);
+    else
+      hipLaunchKernelGGL((crl::k_shared_act<4, 2>), dim3(grid), dim3(block), 0, e->stream, R, P, t,
+                         trace_row, e->key.p, e->delta.p);
+  } else {
+    if (lds_map)
+      hipLaunchKernelGGL((crl::k_shared_act<8, 1>), dim3(grid), dim3(block), lds, e->stream, R, P, t,
+                         trace_row, e->key.p, e->delta.p);
+    else
+      hipLaunchKernelGGL((crl::k_shared_act<8, 2>), dim3(grid), dim3(block), 0, e->stream, R, P, t,
+                         trace_row, e->key.p, e->delta.p);
+  }
+  HIP_TRY(hipGetLastError());
+  return reduce_apply(e, e->Q.p, e->key.p, e->delta.p, e->N);
+}
+
+int check_engine(const crl_engine* e) {
+  if (!e) return fail(CRL_E_ARG, "null engine");
+  hipError_t err = hipSetDevice(e->device);
+  if (err != hipSuccess) return fail(CRL_E_DEVICE, "hipSetDevice(%d): %s", e->device, hipGetErrorString(err));
+  return CRL_OK;
+}
+
+int upload_maps(crl_engine* e) {
+  std::vector<uint32_t> packed((size_t)e->n_maps * e->map_words, 0u);
+  for (int m = 0; m < e->n_maps; ++m)
+    crl::pack_classes(e->h_class.data() + (size_t)m * e->S, e->S,
+                      packed.data() + (size_t)m * e->map_words);
+  HIP_TRY(hipMemcpyAsync(e->map.p, packed.data(), packed.size() * sizeof(uint32_t),
+                         hipMemcpyHostToDevice, e->stream));
+  if (e->cfg.reward_flags & CRL_REWARD_CELLS)
+    HIP_TRY(hipMemcpyAsync(e->cell_reward.p, e->h_cell_reward.data(),
+                           e->h_cell_reward.size() * sizeof(float), hipMemcpyHostToDevice,
+                           e->stream));
+  HIP_TRY(hipStreamSynchronize(e->stream));
+  return CRL_OK;
+}
+
+}  // namespace
+
+extern "C" {
+
+const char* crl_last_error(void) { return g_err.c_str(); }
+const char* crl_version(void) { return CRL_VERSION; }
+
+int crl_device_count(void) {
+  int n = 0;
+  hipError_t e = hipGetDeviceCount(&n);
+  if (e != hipSuccess) return fail(CRL_E_DEVICE, "hipGetDeviceCount: %s", hipGetErrorString(e));
+  return n;
+}
+
+int crl_create(const crl_config* cfg, int device, crl_engine** out) {
+  if (!out) return fail(CRL_E_ARG, "out is null");
+  *out = nullptr;
+  int rc = crl::validate_config(cfg, g_err);
+  if (rc != CRL_OK) return rc;
+  int ndev = 0;
+  hipError_t herr = hipGetDeviceCount(&ndev);
+  if (herr != hipSuccess || ndev <= 0)
+    return fail(CRL_E_DEVICE, "no HIP device available (%s); this engine has no CPU path",
+                herr != hipSuccess ? hipGetErrorString(herr) : "count is 0");
+  if (device < 0 || device >= ndev) return fail(CRL_E_ARG, "device %d out of range [0,%d)", device, ndev);
+  HIP_TRY(hipSetDevice(device));
+
+  crl_engine* e = new (std::nothrow) crl_engine();
+  if (!e) return fail(CRL_E_ALLOC, "host allocation failed");
+  e->cfg = *cfg;
+  e->device = device;
+  e->N = cfg->n_envs;
+  e->W = cfg->width;
+  e->H = cfg->height;
+  e->A = cfg->n_actions;
+  e->S = (size_t)cfg->width * cfg->height;
+  e->K = e->S * e->A;
+  e->n_maps = cfg->map_mode == CRL_MAP_SHARED ? 1 : e->N;
+  e->n_tables = cfg->table_mode == CRL_TABLE_SHARED ? 1 : e->N;
+  e->map_words = (int)((e->S + 15) / 16);
+
+  const size_t N = (size_t)e->N;
+  std::vector<float> eps = crl::build_eps_table(*cfg);
+  e->eps_len = (int)eps.size();
+  const bool cells = (cfg->reward_flags & CRL_REWARD_CELLS) != 0;
+  hipError_t a = hipSuccess;
+  auto acc = [&](hipError_t x) {
+    if (a == hipSuccess) a = x;
+  };
+  acc(e->s.alloc(N));
+  acc(e->ep_step.alloc(N));
+  acc(e->episode.alloc(N));
+  acc(e->start.alloc(N));
+  acc(e->act.alloc(N));
+  acc(e->reward.alloc(N));
+  acc(e->done.alloc(N));
+  acc(e->action.alloc(N));
+  acc(e->map.alloc((size_t)e->n_maps * e->map_words));
+  if (cells) acc(e->cell_reward.alloc((size_t)e->n_maps * e->S));
+  acc(e->Q.alloc((size_t)e->n_tables * e->K));
+  acc(e->eps_tab.alloc(eps.size()));
+  acc(e->tr_s.alloc(N));
+  acc(e->tr_a.alloc(N));
+  acc(e->tr_s2.alloc(N));
+  acc(e->tr_r.alloc(N));
+  acc(e->tr_done.alloc(N));
+  if (cfg->table_mode == CRL_TABLE_SHARED) {
+    acc(e->key.alloc(N));
+    acc(e->delta.alloc(N));
+  }
+  if (a != hipSuccess) {
+    const int code = a == hipErrorOutOfMemory ? CRL_E_ALLOC : CRL_E_DEVICE;
+    delete e;
+    return fail(code, "device allocation failed: %s", hipGetErrorString(a));
+  }
+  try {
+    e->h_class.assign((size_t)e->n_maps * e->S, (uint8_t)CRL_CELL_FREE);
+    if (cells) e->h_cell_reward.assign((size_t)e->n_maps * e->S, cfg->step_reward);
+  } catch (const std::bad_alloc&) {
+    delete e;
+    return fail(CRL_E_ALLOC, "host allocation failed");
+  }
+  auto bail = [&](hipError_t x, const char* what) {
+    delete e;
+    return fail(CRL_E_DEVICE, "%s: %s", what, hipGetErrorString(x));
+  };
+  hipError_t h;
+  if ((h = hipMemsetAsync(e->Q.p, 0, e->Q.n * sizeof(float), e->stream)) != hipSuccess)
+    return bail(h, "clear Q");
+  if ((h = hipMemsetAsync(e->s.p, 0, N * 4, e->stream)) != hipSuccess) return bail(h, "clear s");
+  if ((h = hipMemsetAsync(e->ep_step.p, 0, N * 4, e->stream)) != hipSuccess) return bail(h, "clear");
+  if ((h = hipMemsetAsync(e->episode.p, 0, N * 4, e->stream)) != hipSuccess) return bail(h, "clear");
+  if ((h = hipMemsetAsync(e->start.p, 0, N * 4, e->stream)) != hipSuccess) return bail(h, "clear");
+  if ((h = hipMemsetAsync(e->act.p, 0, N * 4, e->stream)) != hipSuccess) return bail(h, "clear");
+  if ((h = hipMemsetAsync(e->reward.p, 0, N * 4, e->stream)) != hipSuccess) return bail(h, "clear");
+  if ((h = hipMemsetAsync(e->done.p, 0, N, e->stream)) != hipSuccess) return bail(h, "clear");
+  if ((h = hipMemsetAsync(e->action.p, 0, N, e->stream)) != hipSuccess) return bail(h, "clear");
+  if ((h = hipMemsetAsync(e->map.p, 0, e->map.n * 4, e->stream)) != hipSuccess) return bail(h, "clear");
+  if ((h = hipMemcpyAsync(e->eps_tab.p, eps.data(), eps.size() * sizeof(float), hipMemcpyHostToDevice,
+                          e->stream)) != hipSuccess)
+    return bail(h, "upload eps table");
+  if (cells &&
+      (h = hipMemcpyAsync(e->cell_reward.p, e->h_cell_reward.data(), e->h_cell_reward.size() * 4,
+                          hipMemcpyHostToDevice, e->stream)) != hipSuccess)
+    return bail(h, "upload cell rewards");
+  if ((h = hipStreamSynchronize(e->stream)) != hipSuccess) return bail(h, "sync");
+  *out = e;
+  return CRL_OK;
+}
+
+int crl_destroy(crl_engine* e) {
+  if (!e) return CRL_OK;
+  (void)hipSetDevice(e->device);
+  (void)hipStreamSynchronize(e->stream);
+  delete e;
+  return CRL_OK;
+}
+
+int crl_set_stream(crl_engine* e, void* hip_stream) {
+  int rc = check_engine(e);
+  if (rc) return rc;
+  HIP_TRY(hipStreamSynchronize(e->stream));
+  e->stream = reinterpret_cast<hipStream_t>(hip_stream);
+  return CRL_OK;
+}
+
+int crl_sync(crl_engine* e) {
+  int rc = check_engine(e);
+  if (rc) return rc;
+  HIP_TRY(hipStreamSynchronize(e->stream));
+  return CRL_OK;
+}
+
+int crl_set_maps(crl_engine* e, const uint8_t* cell_class, const int32_t* start,
+                 const float* cell_reward) {
+  int rc = check_engine(e);
+  if (rc) return rc;
+  if (!cell_class) return fail(CRL_E_ARG, "cell_class is null");
+  const bool cells = (e->cfg.reward_flags & CRL_REWARD_CELLS) != 0;
+  if (cells && !cell_reward) return fail(CRL_E_ARG, "reward_flags asks for cell rewards but none given");
+  if (!cells && cell_reward) return fail(CRL_E_ARG, "cell rewards given but reward_flags has no CRL_REWARD_CELLS");
+  const size_t total = (size_t)e->n_maps * e->S;
+  for (size_t i = 0; i < total; ++i)
+    if (cell_class[i] > CRL_CELL_WALL) return fail(CRL_E_ARG, "cell_class[%zu] = %d is not a cell class", i, (int)cell_class[i]);
+  if (start)
+    for (int i = 0; i < e->N; ++i)
+      if (start[i] < 0 || (size_t)start[i] >= e->S)
+        return fail(CRL_E_RANGE, "start[%d] = %d outside [0,%zu)", i, start[i], e->S);
+  std::memcpy(e->h_class.data(), cell_class, total);
+  if (cells) std::memcpy(e->h_cell_reward.data(), cell_reward, total * sizeof(float));
+  rc = upload_maps(e);
+  if (rc) return rc;
+  if (start) {
+    HIP_TRY(hipMemcpyAsync(e->start.p, start, (size_t)e->N * 4, hipMemcpyHostToDevice, e->stream));
+    HIP_TRY(hipStreamSynchronize(e->stream));
+  }
+  return crl_reset(e, 0, e->N);
+}
+
+int crl_set_cell(crl_engine* e, int32_t map_index, int32_t cell, int32_t cell_class,
+                 float cell_reward) {
+  int rc = check_engine(e);
+  if (rc) return rc;
+  if (map_index < 0 || map_index >= e->n_maps) return fail(CRL_E_RANGE, "map index %d outside [0,%d)", map_index, e->n_maps);
+  if (cell < 0 || (size_t)cell >= e->S) return fail(CRL_E_RANGE, "cell %d outside [0,%zu)", cell, e->S);
+  if (cell_class < CRL_CELL_FREE || cell_class > CRL_CELL_WALL) return fail(CRL_E_ARG, "%d is not a cell class", cell_class);
+  const size_t at = (size_t)map_index * e->S + cell;
+  e->h_class[at] = (uint8_t)cell_class;
+  const size_t word = (size_t)map_index * e->map_words + (cell >> 4);
+  uint32_t packed = 0;
+  const size_t first = (size_t)map_index * e->S + ((size_t)(cell >> 4) << 4);
+  for (size_t j = 0; j < 16 && ((size_t)(cell >> 4) << 4) + j < e->S; ++j)
+    packed |= (uint32_t)(e->h_class[first + j] & 3u) << (2 * j);
+  HIP_TRY(hipMemcpyAsync(e->map.p + word, &packed, 4, hipMemcpyHostToDevice, e->stream));
+  if (e->cfg.reward_flags & CRL_REWARD_CELLS) {
+    e->h_cell_reward[at] = cell_reward;
+    HIP_TRY(hipMemcpyAsync(e->cell_reward.p + at, &cell_reward, 4, hipMemcpyHostToDevice, e->stream));
+  }
+  HIP_TRY(hipStreamSynchronize(e->stream));
+  return CRL_OK;
+}
+
+int crl_reset(crl_engine* e, int32_t first, int32_t count) {
+  int rc = check_engine(e);
+  if (rc) return rc;
+  if (first < 0 || count < 0 || (int64_t)first + count > e->N)
+    return fail(CRL_E_RANGE, "env range [%d,%d) outside [0,%d)", first, first + count, e->N);
+  if (count == 0) return CRL_OK;
+  hipLaunchKernelGGL(crl::k_reset, dim3((count + 255) / 256), dim3(256), 0, e->stream, e->ptrs(), first,
+                     count);
+  HIP_TRY(hipGetLastError());
+  e->have_transition = false;
+  return CRL_OK;
+}
+
+int crl_step(crl_engine* e, const int32_t* actions) {
+  int rc = check_engine(e);
+  if (rc) return rc;
+  if (actions) {
+    HIP_TRY(hipMemcpyAsync(e->act.p, actions, (size_t)e->N * 4, hipMemcpyHostToDevice, e->stream));
+    // the host buffer may be reused as soon as we return
+    HIP_TRY(hipStreamSynchronize(e->stream));
+  } else if (!e->have_actions) {
+    return fail(CRL_E_STATE, "crl_step(NULL) needs a preceding crl_select");
+  }
+  hipLaunchKernelGGL(crl::k_step, dim3((e->N + 255) / 256), dim3(256), 0, e->stream, e->rules(),
+                     e->ptrs(), e->transition(), e->act.p);
+  HIP_TRY(hipGetLastError());
+  if (e->trace_n > 0 && e->trace_cursor < e->trace_cap) e->trace_cursor += 1;
+  e->have_transition = true;
+  e->have_actions = false;
+  return CRL_OK;
+}
+
+int crl_select(crl_engine* e, int32_t* actions_out) {
+  int rc = check_engine(e);
+  if (rc) return rc;
+  const long long threads = (long long)e->N * e->A;
+  const int grid = (int)((threads + 255) / 256);
+  if (e->A == 4)
+    hipLaunchKernelGGL((crl::k_select<4>), dim3(grid), dim3(256), 0, e->stream, e->rules(), e->ptrs(),
+                       e->t, e->act.p);
+  else
+    hipLaunchKernelGGL((crl::k_select<8>), dim3(grid), dim3(256), 0, e->stream, e->rules(), e->ptrs(),
+                       e->t, e->act.p);
+  HIP_TRY(hipGetLastError());
+  e->have_actions = true;
+  if (actions_out) {
+    HIP_TRY(hipMemcpyAsync(actions_out, e->act.p, (size_t)e->N * 4, hipMemcpyDeviceToHost, e->stream));
+    HIP_TRY(hipStreamSynchronize(e->stream));
+  }
+  return CRL_OK;
+}
+
+int crl_update(crl_engine* e) {
+  int rc = check_engine(e);
+  if (rc) return rc;
+  if (!e->have_transition) return fail(CRL_E_STATE, "crl_update needs a preceding crl_step");
+  const crl::Rules R = e->rules();
+  const int grid = (e->N + 255) / 256;
+  if (e->cfg.table_mode == CRL_TABLE_PER_ENV) {
+    if (e->A == 4)
+      hipLaunchKernelGGL((crl::k_update_per_env<4>), dim3(grid), dim3(256), 0, e->stream, R, e->ptrs(),
+                         e->transition());
+    else
+      hipLaunchKernelGGL((crl::k_update_per_env<8>), dim3(grid), dim3(256), 0, e->stream, R, e->ptrs(),
+                         e->transition());
+    HIP_TRY(hipGetLastError());
+  } else {
+    if (e->A == 4)
+      hipLaunchKernelGGL((crl::k_delta<4>), dim3(grid), dim3(256), 0, e->stream, e->Q.p, e->N, e->tr_s.p,
+                         e->tr_a.p, e->tr_r.p, e->tr_s2.p, e->tr_done.p, R.lr, R.gamma, R.max_mode,
+                         e->key.p, e->delta.p);
+    else
+      hipLaunchKernelGGL((crl::k_delta<8>), dim3(grid), dim3(256), 0, e->stream, e->Q.p, e->N, e->tr_s.p,
+                         e->tr_a.p, e->tr_r.p, e->tr_s2.p, e->tr_done.p, R.lr, R.gamma, R.max_mode,
+                         e->key.p, e->delta.p);
+    HIP_TRY(hipGetLastError());
+    rc = reduce_apply(e, e->Q.p, e->key.p, e->delta.p, e->N);
+    if (rc) return rc;
+  }
+  e->have_transition = false;
+  e->t += 1;
+  return CRL_OK;
+}
+
+int crl_td_update(crl_engine* e, int32_t table, int32_t n, const int32_t* s, const int32_t* a,
+                  const float* r, const int32_t* s_next, const uint8_t* done) {
+  int rc = check_engine(e);
+  if (rc) return rc;
+  if (table < 0 || table >= e->n_tables) return fail(CRL_E_RANGE, "table %d outside [0,%d)", table, e->n_tables);
+  if (n < 0) return fail(CRL_E_ARG, "negative sample count");
+  if (n == 0) return CRL_OK;
+  if (!s || !a || !r || !s_next || !done) return fail(CRL_E_ARG, "null transition array");
+  for (int i = 0; i < n; ++i) {
+    if (s[i] < 0 || (size_t)s[i] >= e->S) return fail(CRL_E_RANGE, "s[%d] = %d outside [0,%zu)", i, s[i], e->S);
+    if (s_next[i] < 0 || (size_t)s_next[i] >= e->S)
+      return fail(CRL_E_RANGE, "s_next[%d] = %d outside [0,%zu)", i, s_next[i], e->S);
+  }
+  const size_t nn = (size_t)n;
+  hipError_t h = hipSuccess;
+  auto acc = [&](hipError_t x) {
+    if (h == hipSuccess) h = x;
+  };
+  acc(e->b_s.ensure(nn));
+  acc(e->b_a.ensure(nn));
+  acc(e->b_s2.ensure(nn));
+  acc(e->b_r.ensure(nn));
+  acc(e->b_done.ensure(nn));
+  acc(e->key.ensure(nn > (size_t)e->N ? nn : (size_t)e->N));
+  acc(e->delta.ensure(nn > (size_t)e->N ? nn : (size_t)e->N));
+  if (h != hipSuccess) return fail(CRL_E_ALLOC, "scratch allocation failed: %s", hipGetErrorString(h));
+  HIP_TRY(hipMemcpyAsync(e->b_s.p, s, nn * 4, hipMemcpyHostToDevice, e->stream));
+  HIP_TRY(hipMemcpyAsync(e->b_a.p, a, nn * 4, hipMemcpyHostToDevice, e->stream));
+  HIP_TRY(hipMemcpyAsync(e->b_r.p, r, nn * 4, hipMemcpyHostToDevice, e->stream));
+  HIP_TRY(hipMemcpyAsync(e->b_s2.p, s_next, nn * 4, hipMemcpyHostToDevice, e->stream));
+  HIP_TRY(hipMemcpyAsync(e->b_done.p, done, nn, hipMemcpyHostToDevice, e->stream));
+  HIP_TRY(hipStreamSynchronize(e->stream));
+  float* Q = e->Q.p + (size_t)table * e->K;
+  const int grid = (n + 255) / 256;
+  if (e->A == 4)
+    hipLaunchKernelGGL((crl::k_delta<4>), dim3(grid), dim3(256), 0, e->stream, Q, n, e->b_s.p, e->b_a.p,
+                       e->b_r.p, e->b_s2.p, e->b_done.p, e->cfg.lr, e->cfg.gamma, e->cfg.max_mode,
+                       e->key.p, e->delta.p);
+  else
+    hipLaunchKernelGGL((crl::k_delta<8>), dim3(grid), dim3(256), 0, e->stream, Q, n, e->b_s.p, e->b_a.p,
+                       e->b_r.p, e->b_s2.p, e->b_done.p, e->cfg.lr, e->cfg.gamma, e->cfg.max_mode,
+                       e->key.p, e->delta.p);
+  HIP_TRY(hipGetLastError());
+  return reduce_apply(e, Q, e->key.p, e->delta.p, n);
+}
+
+int crl_run_fused(crl_engine* e, int32_t n_steps) {
+  int rc = check_engine(e);
+  if (rc) return rc;
+  if (n_steps < 0) return fail(CRL_E_ARG, "negative step count");
+  if (n_steps == 0) return CRL_OK;
+  if (e->cfg.table_mode == CRL_TABLE_PER_ENV) {
+    const FusedPlan p = plan_fused(e);
+    if (e->A == 4)
+      launch_fused_a<4>(e, p, e->t, n_steps);
+    else
+      launch_fused_a<8>(e, p, e->t, n_steps);
+    HIP_TRY(hipGetLastError());
+    if (e->trace_n > 0) {
+      const long long c = (long long)e->trace_cursor + n_steps;
+      e->trace_cursor = c > e->trace_cap ? e->trace_cap : (int)c;
+    }
+  } else {
+    for (int k = 0; k < n_steps; ++k) {
+      rc = shared_step(e, e->t + (uint64_t)k, e->trace_cursor);
+      if (rc) return rc;
+      if (e->trace_n > 0 && e->trace_cursor < e->trace_cap) e->trace_cursor += 1;
+    }
+  }
+  e->t += (uint64_t)n_steps;
+  e->have_transition = false;
+  e->have_actions = false;
+  return CRL_OK;
+}
+
+int crl_get_state(crl_engine* e, int32_t* s, float* reward, uint8_t* done, uint8_t* action,
+                  int32_t* ep_step, int32_t* episode) {
+  int rc = check_engine(e);
+  if (rc) return rc;
+  const size_t N = (size_t)e->N;
+  if (s) HIP_TRY(hipMemcpyAsync(s, e->s.p, N * 4, hipMemcpyDeviceToHost, e->stream));
+  if (reward) HIP_TRY(hipMemcpyAsync(reward, e->reward.p, N * 4, hipMemcpyDeviceToHost, e->stream));
+  if (done) HIP_TRY(hipMemcpyAsync(done, e->done.p, N, hipMemcpyDeviceToHost, e->stream));
+  if (action) HIP_TRY(hipMemcpyAsync(action, e->action.p, N, hipMemcpyDeviceToHost, e->stream));
+  if (ep_step) HIP_TRY(hipMemcpyAsync(ep_step, e->ep_step.p, N * 4, hipMemcpyDeviceToHost, e->stream));
+  if (episode) HIP_TRY(hipMemcpyAsync(episode, e->episode.p, N * 4, hipMemcpyDeviceToHost, e->stream));
+  HIP_TRY(hipStreamSynchronize(e->stream));
+  return CRL_OK;
+}
+
+int crl_set_state(crl_engine* e, const int32_t* s, const int32_t* ep_step, const int32_t* episode) {
+  int rc = check_engine(e);
+  if (rc) return rc;
+  const size_t N = (size_t)e->N;
+  if (s) {
+    for (int i = 0; i < e->N; ++i)
+      if (s[i] < 0 || (size_t)s[i] >= e->S) return fail(CRL_E_RANGE, "s[%d] = %d outside [0,%zu)", i, s[i], e->S);
+    HIP_TRY(hipMemcpyAsync(e->s.p, s, N * 4, hipMemcpyHostToDevice, e->stream));
+  }
+  if (ep_step) HIP_TRY(hipMemcpyAsync(e->ep_step.p, ep_step, N * 4, hipMemcpyHostToDevice, e->stream));
+  if (episode) HIP_TRY(hipMemcpyAsync(e->episode.p, episode, N * 4, hipMemcpyHostToDevice, e->stream));
+  HIP_TRY(hipStreamSynchronize(e->stream));
+  e->have_transition = false;
+  e->have_actions = false;
+  return CRL_OK;
+}
+
+int crl_get_step_count(crl_engine* e, uint64_t* t) {
+  if (!e || !t) return fail(CRL_E_ARG, "null argument");
+  *t = e->t;
+  return CRL_OK;
+}
+
+int crl_set_step_count(crl_engine* e, uint64_t t) {
+  if (!e) return fail(CRL_E_ARG, "null engine");
+  e->t = t;
+  return CRL_OK;
+}
+
+int crl_q_get_range(crl_engine* e, int32_t first_table, int32_t count, float* out) {
+  int rc = check_engine(e);
+  if (rc) return rc;
+  if (!out) return fail(CRL_E_ARG, "out is null");
+  if (first_table < 0 || count < 0 || (int64_t)first_table + count > e->n_tables)
+    return fail(CRL_E_RANGE, "table range [%d,%d) outside [0,%d)", first_table, first_table + count, e->n_tables);
+  HIP_TRY(hipMemcpyAsync(out, e->Q.p + (size_t)first_table * e->K, (size_t)count * e->K * sizeof(float),
+                         hipMemcpyDeviceToHost, e->stream));
+  HIP_TRY(hipStreamSynchronize(e->stream));
+  return CRL_OK;
+}
+
+int crl_q_get(crl_engine* e, int32_t table, float* out) { return crl_q_get_range(e, table, 1, out); }
+
+int crl_q_set(crl_engine* e, int32_t table, const float* in) {
+  int rc = check_engine(e);
+  if (rc) return rc;
+  if (!in) return fail(CRL_E_ARG, "in is null");
+  if (table < 0 || table >= e->n_tables) return fail(CRL_E_RANGE, "table %d outside [0,%d)", table, e->n_tables);
+  HIP_TRY(hipMemcpyAsync(e->Q.p + (size_t)table * e->K, in, e->K * sizeof(float), hipMemcpyHostToDevice,
+                         e->stream));
+  HIP_TRY(hipStreamSynchronize(e->stream));
+  return CRL_OK;
+}
+
+int crl_set_trace(crl_engine* e, int32_t n_envs, int32_t max_steps) {
+  int rc = check_engine(e);
+  if (rc) return rc;
+  if (n_envs < 0 || n_envs > e->N || max_steps < 0) return fail(CRL_E_ARG, "bad trace size");
+  HIP_TRY(hipStreamSynchronize(e->stream));
+  e->trace_n = 0;
+  e->trace_cap = 0;
+  e->trace_cursor = 0;
+  if (n_envs == 0 || max_steps == 0) return CRL_OK;
+  const size_t cells = (size_t)n_envs * max_steps;
+  hipError_t h = hipSuccess;
+  auto acc = [&](hipError_t x) {
+    if (h == hipSuccess) h = x;
+  };
+  acc(e->trace_s.ensure(cells));
+  acc(e->trace_a.ensure(cells));
+  acc(e->trace_r.ensure(cells));
+  acc(e->trace_d.ensure(cells));
+  if (h != hipSuccess) return fail(CRL_E_ALLOC, "trace allocation failed: %s", hipGetErrorString(h));
+  e->trace_n = n_envs;
+  e->trace_cap = max_steps;
+  return CRL_OK;
+}
+
+int crl_get_trace(crl_engine* e, int32_t n_steps, int32_t* s_next, uint8_t* action, float* reward,
+                  uint8_t* done) {
+  int rc = check_engine(e);
+  if (rc) return rc;
+  if (n_steps < 0 || n_steps > e->trace_cursor)
+    return fail(CRL_E_RANGE, "%d steps asked, %d recorded", n_steps, e->trace_cursor);
+  const size_t cells = (size_t)n_steps * e->trace_n;
+  if (cells == 0) return CRL_OK;
+  if (s_next) HIP_TRY(hipMemcpyAsync(s_next, e->trace_s.p, cells * 4, hipMemcpyDeviceToHost, e->stream));
+  if (action) HIP_TRY(hipMemcpyAsync(action, e->trace_a.p, cells, hipMemcpyDeviceToHost, e->stream));
+  if (reward) HIP_TRY(hipMemcpyAsync(reward, e->trace_r.p, cells * 4, hipMemcpyDeviceToHost, e->stream));
+  if (done) HIP_TRY(hipMemcpyAsync(done, e->trace_d.p, cells, hipMemcpyDeviceToHost, e->stream));
+  HIP_TRY(hipStreamSynchronize(e->stream));
+  return CRL_OK;
+}
+
+int crl_set_exploration_stream(crl_engine* e, int32_t n_steps, const float* u, const int32_t* a_rand) {
+  int rc = check_engine(e);
+  if (rc) return rc;
+  HIP_TRY(hipStreamSynchronize(e->stream));
+  e->sup_n = 0;
+  if (!u || n_steps <= 0) return CRL_OK;
+  if (!a_rand) return fail(CRL_E_ARG, "a_rand is null");
+  const size_t cells = (size_t)n_steps * e->N;
+  for (size_t i = 0; i < cells; ++i)
+    if (a_rand[i] < 0 || a_rand[i] >= e->A) return fail(CRL_E_RANGE, "a_rand[%zu] = %d outside [0,%d)", i, a_rand[i], e->A);
+  hipError_t h = e->u_sup.ensure(cells);
+  if (h == hipSuccess) h = e->a_sup.ensure(cells);
+  if (h != hipSuccess) return fail(CRL_E_ALLOC, "stream allocation failed: %s", hipGetErrorString(h));
+  HIP_TRY(hipMemcpyAsync(e->u_sup.p, u, cells * 4, hipMemcpyHostToDevice, e->stream));
+  HIP_TRY(hipMemcpyAsync(e->a_sup.p, a_rand, cells * 4, hipMemcpyHostToDevice, e->stream));
+  HIP_TRY(hipStreamSynchronize(e->stream));
+  e->sup_t0 = e->t;
+  e->sup_n = n_steps;
+  return CRL_OK;
+}
+
+int crl_device_ptr(crl_engine* e, int32_t which, void** out) {
+  if (!e || !out) return fail(CRL_E_ARG, "null argument");
+  switch (which) {
+    case CRL_PTR_S: *out = e->s.p; break;
+    case CRL_PTR_EP_STEP: *out = e->ep_step.p; break;
+    case CRL_PTR_EPISODE: *out = e->episode.p; break;
+    case CRL_PTR_REWARD: *out = e->reward.p; break;
+    case CRL_PTR_DONE: *out = e->done.p; break;
+    case CRL_PTR_ACTION: *out = e->action.p; break;
+    case CRL_PTR_Q: *out = e->Q.p; break;
+    default: return fail(CRL_E_ARG, "unknown pointer id %d", which);
+  }
+  return CRL_OK;
+}
+
+int crl_fused_kernel_info(crl_engine* e, char* name, size_t name_len, int32_t* grid, int32_t* block,
+                          int32_t* lds_bytes) {
+  if (!e) return fail(CRL_E_ARG, "null engine");
+  if (e->cfg.table_mode == CRL_TABLE_PER_ENV) {
+    const FusedPlan p = plan_fused(e);
+    if (name && name_len) snprintf(name, name_len, "%s", p.name);
+    if (grid) *grid = p.grid;
+    if (block) *block = p.block;
+    if (lds_bytes) *lds_bytes = (int32_t)p.lds;
+  } else {
+    if (name && name_len) snprintf(name, name_len, "k_shared_act+k_reduce_apply");
+    if (grid) *grid = (e->N + 255) / 256;
+    if (block) *block = 256;
+    if (lds_bytes) *lds_bytes = e->map_words * 4;
+  }
+  return CRL_OK;
+}
+
+}  // extern "C"

@@ -1,0 +1,247 @@
+/*
+ * crl.h - C ABI of the MI355X (gfx950) batched grid-world + tabular Q-learning engine.
+ *
+ * Everything here is `extern "C"`, plain pointers and sizes.  Every function
+ * returns an int status (CRL_OK or a negative CRL_E_* code) unless stated;
+ * `crl_last_error()` gives the text of the calling thread's last failure.
+ * Nothing throws across this boundary.  Host buffers belong to the caller,
+ * device buffers to the engine.  Calls on one engine must be serialised by
+ * the caller; there is no CPU fallback: without a usable HIP device
+ * `crl_create` fails with CRL_E_DEVICE.
+ *
+ * Citations name the file:line of life423/CudaRL-Arena that the entry point
+ * replaces.  State index is s = y*W + x and the table layout is
+ * Q[s*A + a], fp32 (src/kernels.cu:96, src/q_learning.cu:196).
+ *
+ * Actions (src/kernels.cu:15-23): 0 = up (dy-1), 1 = right (dx+1),
+ * 2 = down (dy+1), 3 = left (dx-1); any other value is "no move".  With
+ * n_actions == 8 the diagonals follow: 4 = up-right, 5 = down-right,
+ * 6 = down-left, 7 = up-left.
+ */
+#ifndef CRL_H
+#define CRL_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define CRL_VERSION "0.1.0" /* src/python_bindings.cpp:24 */
+
+/* status codes */
+enum {
+  CRL_OK = 0,
+  CRL_E_ARG = -1,      /* bad argument / inconsistent sizes               */
+  CRL_E_DEVICE = -2,   /* no HIP device, or a HIP call failed             */
+  CRL_E_ALLOC = -3,    /* device or host allocation failed                */
+  CRL_E_STATE = -4,    /* call not valid in the engine's current state    */
+  CRL_E_RANGE = -5     /* index out of range                              */
+};
+
+/* cell classes; thresholds on the reference's float grid are
+ * FREE [0,0.99), GOAL >= 0.99, TRAP (-1,0), WALL <= -1 (src/kernels.cu:30-63) */
+enum { CRL_CELL_FREE = 0, CRL_CELL_GOAL = 1, CRL_CELL_TRAP = 2, CRL_CELL_WALL = 3 };
+
+enum { CRL_TABLE_PER_ENV = 0, CRL_TABLE_SHARED = 1 };
+enum { CRL_MAP_PER_ENV = 0, CRL_MAP_SHARED = 1 };
+
+/* max over the next row: TRUE_MAX follows src/gpu/kernels.cu:35-45,
+ * ZERO_FLOOR follows src/kernels.cu:101-110 (max seeded with 0.0f). */
+enum { CRL_MAX_TRUE = 0, CRL_MAX_ZERO_FLOOR = 1 };
+
+/* goal test: TARGET follows src/kernels.cu:50-58 (class of the in-bounds
+ * target cell), RESULT follows src/environment.cu:43 (class of the cell the
+ * agent stands on after the move, so an out-of-bounds bump on the goal
+ * re-fires it). */
+enum { CRL_GOAL_ON_TARGET = 0, CRL_GOAL_ON_RESULT = 1 };
+
+/* exploration schedules (src/train.py:100-108,140-141) */
+enum {
+  CRL_EPS_FIXED = 0,            /* eps0 for ever                                   */
+  CRL_EPS_STEP_MULT = 1,        /* eps0 * decay^t, t = global step (the reference) */
+  CRL_EPS_EPISODE_MULT = 2,     /* eps0 * decay^episode, per env                   */
+  CRL_EPS_EPISODE_LINEAR = 3    /* eps0 -> eps_end linearly over eps_span episodes */
+};
+
+/* reward_flags bits */
+enum {
+  CRL_REWARD_CELLS = 1,      /* a per-cell fp32 array gives the goal / trap rewards   */
+  CRL_REWARD_BASE_CELLS = 2  /* ... and also the plain-step reward (cell stood on)    */
+};
+
+typedef struct crl_config {
+  uint32_t struct_size;  /* sizeof(crl_config), checked                            */
+  int32_t n_envs;        /* N >= 1                                                 */
+  int32_t width, height; /* W, H >= 1; S = W*H                                      */
+  int32_t n_actions;     /* A: 4 or 8                                              */
+  int32_t table_mode;    /* CRL_TABLE_*                                            */
+  int32_t map_mode;      /* CRL_MAP_*                                              */
+  int32_t max_mode;      /* CRL_MAX_*                                              */
+  int32_t goal_mode;     /* CRL_GOAL_*                                             */
+  int32_t auto_reset;    /* 1: an env that is done or has used episode_len steps
+                            restarts from its start cell; 0: done is sticky
+                            (src/environment.cu:44-46 never clears it)             */
+  int32_t episode_len;   /* T; 0 = no limit                                        */
+  float lr, gamma;       /* src/q_learning.cuh:18-19                               */
+  float step_reward;     /* -0.01f (src/kernels.cu:46)                             */
+  float goal_reward;     /*  1.0f  (src/kernels.cu:56)                             */
+  float trap_reward;     /* bump penalty of a TRAP cell when no cell array is set   */
+  int32_t reward_flags;  /* CRL_REWARD_* bits                                      */
+  int32_t eps_mode;      /* CRL_EPS_*                                              */
+  float eps0, eps_decay, eps_end;
+  int32_t eps_span;      /* table length for the STEP/EPISODE schedules            */
+  uint64_t seed;         /* Philox4x32-10 key                                      */
+} crl_config;
+
+typedef struct crl_engine crl_engine;
+
+/* -- life cycle ---------------------------------------------------------- */
+
+const char* crl_last_error(void);
+const char* crl_version(void);
+/* number of HIP devices, or a negative status */
+int crl_device_count(void);
+
+/* Replaces the constructors Environment::Environment (src/environment.cu:50-77)
+ * and CudaQLearning::CudaQLearning (src/q_learning.cu:6-94): allocates the SoA
+ * state, the map and the zero-initialised table(s) on device `device`.  All
+ * envs start on cell 0 of an all-FREE map until crl_set_maps is called. */
+int crl_create(const crl_config* cfg, int device, crl_engine** out);
+/* Replaces ~Environment / ~CudaQLearning (src/environment.cu:79-100,
+ * src/q_learning.cu:96-106).  NULL is allowed. */
+int crl_destroy(crl_engine* e);
+/* Use `hip_stream` (a hipStream_t, NULL = the null stream) for all later work. */
+int crl_set_stream(crl_engine* e, void* hip_stream);
+int crl_sync(crl_engine* e);
+
+/* -- maps ------------------------------------------------------------------ */
+
+/* Replaces Environment::initializeGrid + the H2D grid copy
+ * (src/environment.cu:60-74,138-147).  cell_class: n_maps*S bytes of CRL_CELL_*
+ * (n_maps = N, or 1 when map_mode is SHARED); start: N cell indices (NULL keeps
+ * the current ones); cell_reward: n_maps*S floats, required iff reward_flags has
+ * CRL_REWARD_CELLS.  Also resets every env (as crl_reset(e,0,N)). */
+int crl_set_maps(crl_engine* e, const uint8_t* cell_class, const int32_t* start,
+                 const float* cell_reward);
+/* Edit one cell; gives EnvironmentBridge::addObstacle/setGoal/addTrap
+ * (src/environment_bridge.cu:53-78, print-only upstream) an effect. */
+int crl_set_cell(crl_engine* e, int32_t map_index, int32_t cell, int32_t cell_class,
+                 float cell_reward);
+/* Classify the reference's float grid (thresholds of src/kernels.cu:30-63):
+ * out_class[i] in CRL_CELL_*, out_reward[i] = 1.0f for GOAL, v for TRAP,
+ * step_reward otherwise.  Host only. */
+int crl_classify_grid(const float* grid, size_t n, float step_reward, uint8_t* out_class,
+                      float* out_reward);
+
+/* -- the hot path ---------------------------------------------------------- */
+
+/* Environment::reset (src/environment.cu:102-111; kernel :6-14): envs
+ * [first, first+count) go to their start cell, reward 0, done false,
+ * episode step 0.  The episode counter is not changed. */
+int crl_reset(crl_engine* e, int32_t first, int32_t count);
+
+/* Environment::step (src/environment.cu:113-125) with the wall / trap / goal
+ * rules of step_environment_kernel (src/kernels.cu:13-66), for all N envs.
+ * `actions` = N host int32 (NULL: use the actions the last crl_select left on
+ * the device).  Records the transition (s, a, r, s', done) for crl_update. */
+int crl_step(crl_engine* e, const int32_t* actions);
+
+/* Epsilon-greedy selection (src/train.py:100-108) with the greedy branch of
+ * CudaQLearning::get_best_action (src/q_learning.cu:191-209: lowest index wins
+ * ties).  The uniforms come from Philox4x32-10 keyed (seed; env, step) unless an
+ * exploration stream was supplied.  actions_out: N host int32 or NULL. */
+int crl_select(crl_engine* e, int32_t* actions_out);
+
+/* TD update of the transition recorded by the last crl_step
+ * (src/gpu/kernels.cu:7-54); advances the global step counter by one. */
+int crl_update(crl_engine* e);
+
+/* CudaQLearning::update_batch (src/q_learning.cu:108-174): n explicit
+ * transitions on table `table` (0 for a shared table, the env index
+ * otherwise).  All reads see the table as it was before the call; deltas that
+ * hit the same (s,a) are summed in sample order and then applied.  Host arrays. */
+int crl_td_update(crl_engine* e, int32_t table, int32_t n, const int32_t* s, const int32_t* a,
+                  const float* r, const int32_t* s_next, const uint8_t* done);
+
+/* n_steps of select -> step -> update for every env, fused on the device
+ * (the loop body of src/train.py:198-222).  Same results as n_steps rounds of
+ * crl_select; crl_step(NULL); crl_update. */
+int crl_run_fused(crl_engine* e, int32_t n_steps);
+
+/* Environment getters (src/environment.h:26-37) for all envs; any pointer may
+ * be NULL.  s = cell the env acts from next, reward/done/action = last step. */
+int crl_get_state(crl_engine* e, int32_t* s, float* reward, uint8_t* done, uint8_t* action,
+                  int32_t* ep_step, int32_t* episode);
+/* Restore a saved state (checkpoint / resume; no reference counterpart beyond
+ * get/set_q_table).  Any pointer may be NULL. */
+int crl_set_state(crl_engine* e, const int32_t* s, const int32_t* ep_step,
+                  const int32_t* episode);
+/* global step counter t (number of updates so far) */
+int crl_get_step_count(crl_engine* e, uint64_t* t);
+int crl_set_step_count(crl_engine* e, uint64_t t);
+
+/* CudaQLearning::get_q_table / set_q_table (src/q_learning.cu:176-189):
+ * S*A floats of table `table`. */
+int crl_q_get(crl_engine* e, int32_t table, float* out);
+int crl_q_set(crl_engine* e, int32_t table, const float* in);
+/* several consecutive tables in one copy */
+int crl_q_get_range(crl_engine* e, int32_t first_table, int32_t count, float* out);
+
+/* -- test hooks ------------------------------------------------------------ */
+
+/* Record (s', action, reward, done) of envs [0, n_envs) for the next
+ * `max_steps` steps run by crl_run_fused / crl_step.  n_envs = 0 turns it off. */
+int crl_set_trace(crl_engine* e, int32_t n_envs, int32_t max_steps);
+/* Copy out `n_steps` recorded steps, arrays [n_steps][n_trace_envs]. */
+int crl_get_trace(crl_engine* e, int32_t n_steps, int32_t* s_next, uint8_t* action,
+                  float* reward, uint8_t* done);
+/* Supply the exploration stream instead of Philox: u[n_steps][N] in [0,1) and
+ * a_rand[n_steps][N] in [0,A), consumed by steps t0 .. t0+n_steps-1 where t0 is
+ * the step counter at the time of this call.  NULL u removes it. */
+int crl_set_exploration_stream(crl_engine* e, int32_t n_steps, const float* u,
+                               const int32_t* a_rand);
+
+/* raw device pointers of the SoA state for zero-copy consumers; index with
+ * CRL_PTR_*.  Valid until crl_destroy. */
+enum {
+  CRL_PTR_S = 0, CRL_PTR_EP_STEP = 1, CRL_PTR_EPISODE = 2, CRL_PTR_REWARD = 3,
+  CRL_PTR_DONE = 4, CRL_PTR_ACTION = 5, CRL_PTR_Q = 6, CRL_PTR_COUNT = 7
+};
+int crl_device_ptr(crl_engine* e, int32_t which, void** out);
+
+/* name and launch geometry of the kernel crl_run_fused uses for this engine */
+int crl_fused_kernel_info(crl_engine* e, char* name, size_t name_len, int32_t* grid,
+                          int32_t* block, int32_t* lds_bytes);
+
+/* -- host-side helpers (no device needed) ----------------------------------- */
+
+/* Philox4x32-10 (Salmon et al. 2011), exposed for tests. */
+void crl_philox4x32_10(const uint32_t ctr[4], const uint32_t key[2], uint32_t out[4]);
+/* the two exploration draws of (seed, env, step t): u in [0,1), a in [0,A) */
+void crl_explore_draw(uint64_t seed, uint32_t env, uint64_t t, int32_t n_actions, float* u,
+                      int32_t* a_rand);
+/* epsilon table the engine would build for cfg (length written to *len, at
+ * most cap entries copied) */
+int crl_eps_table(const crl_config* cfg, float* out, int32_t cap, int32_t* len);
+
+/* Synthetic maps (no reference counterpart: src/environment.cu:140 seeds from
+ * the wall clock).  Cells are WALL with probability p_wall, then TRAP with
+ * probability p_trap among the rest; one GOAL per map and N start cells drawn
+ * uniformly among the FREE cells.  n_maps = 1 gives a shared map with n_envs
+ * starts.  All draws are Philox4x32-10 from `seed`. */
+int crl_gen_maps_bernoulli(uint64_t seed, int32_t n_maps, int32_t n_envs, int32_t width,
+                           int32_t height, float p_wall, float p_trap, uint8_t* cell_class,
+                           int32_t* start);
+/* Value-noise maps (lattice pitch `pitch`, smoothstep-bilinear): the
+ * `wall_frac` highest-valued cells are WALL; cell_reward = sigma * N(0,1) with
+ * goal_bonus added on the GOAL cell. */
+int crl_gen_maps_noise(uint64_t seed, int32_t n_maps, int32_t width, int32_t height,
+                       int32_t pitch, float wall_frac, float sigma, float goal_bonus,
+                       uint8_t* cell_class, int32_t* start, float* cell_reward);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* CRL_H */

@@ -1,0 +1,461 @@
+/*
+ * crl_oracle.c - CPU restatement of the CudaRL-Arena hot path.
+ *
+ * THIS IS TEST INFRASTRUCTURE.  It is the checker the HIP engine is compared
+ * against; only tests/, __graft_entry__.smoke() and bench.py's cpu_baseline
+ * leg may load it.  The product never calls it.
+ *
+ * Scalar C, one env at a time, no vectorisation tricks.  Each function cites
+ * the file:line of life423/CudaRL-Arena it follows.  Compile with
+ * -ffp-contract=off: the two fused multiply-adds of the TD update are written
+ * as explicit fmaf so that every compiler produces the same bits.
+ *
+ * What pins each function (see tests/test_oracle_*.py):
+ *   orc_reset_xy, orc_step_e1     the Catch2 cases of tests/test_environment.cpp
+ *   orc_step_e2, orc_classify     no reference test exists: pinned by the
+ *                                 invariants of src/kernels.cu:13-66 on a
+ *                                 brute-forced grid holding every cell class and
+ *                                 the threshold edge values, and by reducing to
+ *                                 orc_step_e1 on obstacle-free grids
+ *   orc_step_cls                  equality with orc_step_e2 on classified grids
+ *   orc_argmax                    src/q_learning.cu:191-209 tie rule, numpy argmax
+ *   orc_td_*                      closed forms (geometric series), float64 numpy
+ *                                 restatement of src/train.py:127-138
+ *   orc_philox4x32_10             Random123 known-answer vectors
+ *   orc_run + eps schedule        training.log:24931-24953 (returns -5.00 / -10.00,
+ *                                 epsilon 0.082, 0.007, 0.001)
+ *   ordered reduction (shared)    defined here, not by the reference: brute force
+ *                                 against a dictionary-of-lists summation
+ */
+#include <math.h>
+#include <stdint.h>
+#include <stdlib.h>
+#include <string.h>
+
+/* same field order as the engine's configuration block so that one ctypes
+ * structure serves both; declared independently on purpose */
+typedef struct orc_config {
+  uint32_t struct_size;
+  int32_t n_envs;
+  int32_t width, height;
+  int32_t n_actions;
+  int32_t table_mode; /* 0 per env, 1 shared */
+  int32_t map_mode;   /* 0 per env, 1 shared */
+  int32_t max_mode;   /* 0 true max, 1 zero floor */
+  int32_t goal_mode;  /* 0 on target cell, 1 on resulting cell */
+  int32_t auto_reset;
+  int32_t episode_len;
+  float lr, gamma;
+  float step_reward, goal_reward, trap_reward;
+  int32_t reward_flags; /* 1 cell array for goal/trap, 2 also for the base */
+  int32_t eps_mode;     /* 0 fixed, 1 step mult, 2 episode mult, 3 episode linear */
+  float eps0, eps_decay, eps_end;
+  int32_t eps_span;
+  uint64_t seed;
+} orc_config;
+
+enum { FREE = 0, GOAL = 1, TRAP = 2, WALL = 3 };
+
+/* ---- Philox4x32-10 (Salmon, Moraes, Dror, Shaw, SC'11) ------------------- */
+
+void orc_philox4x32_10(const uint32_t ctr[4], const uint32_t key[2], uint32_t out[4]) {
+  uint32_t c0 = ctr[0], c1 = ctr[1], c2 = ctr[2], c3 = ctr[3];
+  uint32_t k0 = key[0], k1 = key[1];
+  for (int round = 0; round < 10; ++round) {
+    uint64_t p0 = (uint64_t)0xD2511F53u * c0;
+    uint64_t p1 = (uint64_t)0xCD9E8D57u * c2;
+    uint32_t n0 = (uint32_t)(p1 >> 32) ^ c1 ^ k0;
+    uint32_t n1 = (uint32_t)p1;
+    uint32_t n2 = (uint32_t)(p0 >> 32) ^ c3 ^ k1;
+    uint32_t n3 = (uint32_t)p0;
+    c0 = n0; c1 = n1; c2 = n2; c3 = n3;
+    k0 += 0x9E3779B9u;
+    k1 += 0xBB67AE85u;
+  }
+  out[0] = c0; out[1] = c1; out[2] = c2; out[3] = c3;
+}
+
+/* Exploration draws of (seed, env, step t).  Counter = (env, stream 0,
+ * block lo, block hi) with block = t >> 1; even steps take words 0,1 and odd
+ * steps words 2,3.  u = top 24 bits / 2^24; a = (word * A) >> 32. */
+void orc_explore_draw(uint64_t seed, uint32_t env, uint64_t t, int32_t A, float* u,
+                      int32_t* a_rand) {
+  uint64_t blk = t >> 1;
+  uint32_t ctr[4] = {env, 0u, (uint32_t)blk, (uint32_t)(blk >> 32)};
+  uint32_t key[2] = {(uint32_t)seed, (uint32_t)(seed >> 32)};
+  uint32_t w[4];
+  orc_philox4x32_10(ctr, key, w);
+  uint32_t w0 = (t & 1) ? w[2] : w[0];
+  uint32_t w1 = (t & 1) ? w[3] : w[1];
+  *u = (float)(w0 >> 8) * (1.0f / 16777216.0f);
+  *a_rand = (int32_t)(((uint64_t)w1 * (uint32_t)A) >> 32);
+}
+
+/* ---- E0: reset (src/kernels.cu:3-11, src/environment.cu:6-14) ------------ */
+
+void orc_reset_xy(int W, int H, int* x, int* y, float* reward, int* done) {
+  *x = W / 2;
+  *y = H / 2;
+  *reward = 0.0f;
+  *done = 0;
+}
+
+static void action_delta(int action, int* dx, int* dy) {
+  *dx = 0;
+  *dy = 0;
+  switch (action) { /* src/kernels.cu:18-23; 4..7 are this build's diagonals */
+    case 0: *dy = -1; break;
+    case 1: *dx = 1; break;
+    case 2: *dy = 1; break;
+    case 3: *dx = -1; break;
+    case 4: *dx = 1; *dy = -1; break;
+    case 5: *dx = 1; *dy = 1; break;
+    case 6: *dx = -1; *dy = 1; break;
+    case 7: *dx = -1; *dy = -1; break;
+    default: break;
+  }
+}
+
+/* ---- E1: step without obstacles (src/environment.cu:17-48) --------------- */
+
+void orc_step_e1(int W, int H, int* x, int* y, float* reward, int* done, int action) {
+  int dx = 0, dy = 0;
+  if (action >= 0 && action <= 3) action_delta(action, &dx, &dy);
+  int nx = *x + dx, ny = *y + dy;
+  if (nx >= 0 && nx < W && ny >= 0 && ny < H) {
+    *x = nx;
+    *y = ny;
+  }
+  *reward = -0.01f;
+  if (*x == W - 1 && *y == 0) {
+    *reward = 1.0f;
+    *done = 1; /* never cleared: sticky */
+  }
+}
+
+/* ---- E2: step on a float grid (src/kernels.cu:13-66) --------------------- */
+
+void orc_step_e2(const float* grid, int W, int H, int* x, int* y, float* reward, int* done,
+                 int action) {
+  int dx = 0, dy = 0;
+  if (action >= 0 && action <= 3) action_delta(action, &dx, &dy);
+  int nx = *x + dx, ny = *y + dy;
+  int in = nx >= 0 && nx < W && ny >= 0 && ny < H;
+  int idx = ny * W + nx;
+  int obstacle = 0;
+  if (in) obstacle = grid[idx] < 0.0f; /* :34 */
+  if (in && !obstacle) {                /* :38-43 */
+    *x = nx;
+    *y = ny;
+  }
+  *reward = -0.01f; /* :46 */
+  if (in) {
+    float v = grid[idx];
+    if (v >= 0.99f) { /* :55-58 */
+      *reward = 1.0f;
+      *done = 1;
+    } else if (v < 0.0f && v > -1.0f) { /* :60-62 */
+      *reward = v;
+    }
+  }
+}
+
+/* cell class of a float cell value, thresholds of src/kernels.cu:34,55,60 */
+uint8_t orc_classify(float v) {
+  if (v >= 0.99f) return GOAL;
+  if (v < 0.0f && v > -1.0f) return TRAP;
+  if (v < 0.0f) return WALL; /* v <= -1 */
+  return FREE;               /* [0, 0.99), and NaN: no comparison holds */
+}
+
+/* ---- generalised step on cell classes ------------------------------------ */
+/* cls / cr describe ONE map of S cells.  Returns the hit flag (goal reached
+ * in this step); *s is replaced by the cell after the move. */
+int orc_step_cls(const orc_config* c, const uint8_t* cls, const float* cr, int32_t* s,
+                 int action, float* reward) {
+  const int W = c->width, H = c->height;
+  int x = *s % W, y = *s / W;
+  int dx = 0, dy = 0;
+  if (action >= 0 && action < c->n_actions) action_delta(action, &dx, &dy);
+  int nx = x + dx, ny = y + dy;
+  int in = nx >= 0 && nx < W && ny >= 0 && ny < H;
+  int tgt = ny * W + nx;
+  int k = in ? cls[tgt] : FREE;
+  int moved = in && k < TRAP; /* v < 0 blocks: traps and walls */
+  int s2 = moved ? tgt : *s;
+  const int cells = (c->reward_flags & 1) != 0;
+  float r = (cells && (c->reward_flags & 2)) ? cr[s2] : c->step_reward;
+  int hit = 0;
+  if (c->goal_mode == 0) {
+    if (in) {
+      if (k == GOAL) {
+        r = cells ? cr[tgt] : c->goal_reward;
+        hit = 1;
+      } else if (k == TRAP) {
+        r = cells ? cr[tgt] : c->trap_reward;
+      }
+    }
+  } else { /* goal test on the resulting cell (src/environment.cu:43) */
+    if (in && k == TRAP) r = cells ? cr[tgt] : c->trap_reward;
+    if (cls[s2] == GOAL) {
+      r = cells ? cr[s2] : c->goal_reward;
+      hit = 1;
+    }
+  }
+  *s = s2;
+  *reward = r;
+  return hit;
+}
+
+/* ---- S2: greedy argmax (src/q_learning.cu:191-209) ----------------------- */
+
+int orc_argmax(const float* row, int A) {
+  int best = 0;
+  float bv = row[0];
+  for (int a = 1; a < A; ++a) {
+    if (row[a] > bv) {
+      bv = row[a];
+      best = a;
+    }
+  }
+  return best;
+}
+
+/* ---- S1: epsilon-greedy (src/train.py:100-108) --------------------------- */
+
+int orc_select(const float* row, int A, float eps, float u, int a_rand) {
+  if (u < eps) return a_rand;
+  return orc_argmax(row, A);
+}
+
+/* ---- Q1 / Q2: TD target and update --------------------------------------- */
+
+/* max over the next row; mode 0 = true max (src/gpu/kernels.cu:35-45),
+ * mode 1 = seeded with 0.0f (src/kernels.cu:101-110) */
+float orc_next_max(const float* next_row, int A, int done, int mode) {
+  float m = 0.0f;
+  if (!done) {
+    for (int a = 0; a < A; ++a) {
+      float q = next_row[a];
+      if (mode == 0)
+        m = (a == 0) ? q : fmaxf(m, q);
+      else
+        m = fmaxf(m, q);
+    }
+  }
+  return m;
+}
+
+/* new value of Q[s,a] (src/gpu/kernels.cu:47-52), with the two contractions a
+ * GPU compiler makes written out */
+float orc_td_value(float q, float r, float m, float lr, float gamma) {
+  float target = fmaf(gamma, m, r);
+  return fmaf(lr, target - q, q);
+}
+
+/* delta of one sample for the summed (batch / shared table) form */
+float orc_td_delta(float q, float r, float m, float lr, float gamma) {
+  float target = fmaf(gamma, m, r);
+  return lr * (target - q);
+}
+
+/* one in-place sample on one table (src/gpu/kernels.cu:7-54, one thread) */
+void orc_td_update_one(float* Q, int A, int s, int a, float r, int s2, int done, float lr,
+                       float gamma, int mode) {
+  float m = orc_next_max(Q + (size_t)s2 * A, A, done, mode);
+  Q[(size_t)s * A + a] = orc_td_value(Q[(size_t)s * A + a], r, m, lr, gamma);
+}
+
+/* Batch on one table of K = S*A entries: every read sees the table before the
+ * call; deltas of equal (s,a) are added in sample order, left to right,
+ * starting from +0.0f; then Q[k] = Q[k] + sum[k] for every k.  (The
+ * reference's kernel races on duplicates, src/kernels.cu:114; this is the
+ * build's deterministic rule and equals the reference up to one rounding when
+ * every (s,a) is unique and no written row is another sample's next row.) */
+int orc_td_update_batch(float* Q, int S, int A, int n, const int32_t* s, const int32_t* a,
+                        const float* r, const int32_t* s2, const uint8_t* done, float lr,
+                        float gamma, int mode) {
+  size_t K = (size_t)S * A;
+  float* sum = (float*)calloc(K, sizeof(float));
+  if (!sum) return -3;
+  for (int i = 0; i < n; ++i) {
+    float m = orc_next_max(Q + (size_t)s2[i] * A, A, done[i], mode);
+    size_t k = (size_t)s[i] * A + a[i];
+    sum[k] = sum[k] + orc_td_delta(Q[k], r[i], m, lr, gamma);
+  }
+  for (size_t k = 0; k < K; ++k) Q[k] = Q[k] + sum[k];
+  free(sum);
+  return 0;
+}
+
+/* ---- epsilon schedule ------------------------------------------------------ */
+/* src/train.py:140-141 multiplies a Python float (double) once per update;
+ * the table holds those doubles rounded to fp32.  Returns the length. */
+int orc_eps_table(const orc_config* c, float* out, int cap) {
+  int len = 1;
+  if (c->eps_mode == 0) {
+    if (cap > 0) out[0] = c->eps0;
+    return 1;
+  }
+  if (c->eps_mode == 1 || c->eps_mode == 2) {
+    len = c->eps_span > 0 ? c->eps_span : 1;
+    double e = (double)c->eps0;
+    for (int i = 0; i < len; ++i) {
+      if (i < cap) out[i] = (float)e;
+      e *= (double)c->eps_decay;
+    }
+    return len;
+  }
+  /* linear: span+1 entries, the last is eps_end */
+  int span = c->eps_span > 0 ? c->eps_span : 1;
+  len = span + 1;
+  for (int i = 0; i < len; ++i) {
+    double e = (double)c->eps0 + ((double)c->eps_end - (double)c->eps0) * (double)i / (double)span;
+    if (i < cap) out[i] = (float)e;
+  }
+  return len;
+}
+
+static float eps_at(const orc_config* c, const float* tab, int len, uint64_t t, int32_t episode) {
+  if (c->eps_mode == 0) return c->eps0;
+  uint64_t i = (c->eps_mode == 1) ? t : (uint64_t)(episode < 0 ? 0 : episode);
+  if (i >= (uint64_t)len) i = (uint64_t)len - 1;
+  return tab[i];
+}
+
+/* ---- D1: the driver loop (src/train.py:198-222), batched ------------------ */
+
+static int eps_cap(const orc_config* c) {
+  if (c->eps_mode == 1 || c->eps_mode == 2) return c->eps_span > 0 ? c->eps_span : 1;
+  if (c->eps_mode == 3) return (c->eps_span > 0 ? c->eps_span : 1) + 1;
+  return 1;
+}
+
+/* One env, one step: select (src/train.py:200) -> step (:201) -> update (:205).
+ * q is the env's table (or the shared one); with sum != NULL the delta is
+ * accumulated there instead of being applied.  Returns s' before any restart. */
+static int32_t env_step(const orc_config* c, float eps, float u, int32_t ar, const uint8_t* m_cls,
+                        const float* m_cr, float* q, float* sum, int32_t start, int32_t* s,
+                        int32_t* ep_step, int32_t* episode, float* reward, uint8_t* done,
+                        uint8_t* action) {
+  const int A = c->n_actions;
+  int32_t s0 = *s;
+  int a = orc_select(q + (size_t)s0 * A, A, eps, u, ar);
+  int32_t s2 = s0;
+  float r;
+  int hit = orc_step_cls(c, m_cls, m_cr, &s2, a, &r);
+  int d = hit || (!c->auto_reset && *done);
+  float mx = orc_next_max(q + (size_t)s2 * A, A, d, c->max_mode);
+  size_t key = (size_t)s0 * A + a;
+  if (sum)
+    sum[key] = sum[key] + orc_td_delta(q[key], r, mx, c->lr, c->gamma);
+  else
+    q[key] = orc_td_value(q[key], r, mx, c->lr, c->gamma);
+  *ep_step += 1;
+  *reward = r;
+  *done = (uint8_t)d;
+  *action = (uint8_t)a;
+  if (c->auto_reset && (d || (c->episode_len > 0 && *ep_step >= c->episode_len))) {
+    *s = start;
+    *ep_step = 0;
+    *episode += 1;
+  } else {
+    *s = s2;
+  }
+  return s2;
+}
+
+/*
+ * n_steps of select -> step -> update for all envs, starting at global step
+ * t0.  cls/cr: n_maps maps (1 when map_mode is shared); Q: N tables or one.
+ * s, ep_step, episode, reward, done, action: per-env state, in and out.
+ * u_sup/a_sup (optional, [n_steps][N]) replace the Philox draws.
+ * Trace arrays (optional) are [n_steps][trace_n].
+ *
+ * Shared table: every env of a step reads the table as it was before the
+ * step; the deltas are then summed per (s,a) in env order, left to right from
+ * +0.0f, and Q[k] = Q[k] + sum[k] for every k.
+ */
+int orc_run(const orc_config* c, const uint8_t* cls, const float* cr, const int32_t* start,
+            float* Q, int32_t* s, int32_t* ep_step, int32_t* episode, float* reward,
+            uint8_t* done, uint8_t* action, uint64_t t0, int32_t n_steps, const float* u_sup,
+            const int32_t* a_sup, int32_t trace_n, int32_t* tr_s, uint8_t* tr_a, float* tr_r,
+            uint8_t* tr_d) {
+  const int N = c->n_envs, A = c->n_actions;
+  const size_t S = (size_t)c->width * c->height;
+  const size_t K = S * A;
+  const int shared = c->table_mode == 1;
+  int cap = eps_cap(c);
+  float* tab = (float*)malloc((size_t)cap * sizeof(float));
+  float* sum = shared ? (float*)malloc(K * sizeof(float)) : NULL;
+  if (!tab || (shared && !sum)) {
+    free(tab);
+    free(sum);
+    return -3;
+  }
+  int len = orc_eps_table(c, tab, cap);
+
+  for (int k = 0; k < n_steps; ++k) {
+    uint64_t t = t0 + (uint64_t)k;
+    if (shared)
+      for (size_t kk = 0; kk < K; ++kk) sum[kk] = 0.0f;
+    for (int i = 0; i < N; ++i) {
+      size_t mo = c->map_mode == 1 ? 0 : (size_t)i * S;
+      float u;
+      int32_t ar;
+      if (u_sup) {
+        u = u_sup[(size_t)k * N + i];
+        ar = a_sup[(size_t)k * N + i];
+      } else {
+        orc_explore_draw(c->seed, (uint32_t)i, t, A, &u, &ar);
+      }
+      float eps = eps_at(c, tab, len, t, episode[i]);
+      int32_t s2 = env_step(c, eps, u, ar, cls + mo, cr ? cr + mo : NULL,
+                            Q + (shared ? 0 : (size_t)i * K), sum, start[i], &s[i], &ep_step[i],
+                            &episode[i], &reward[i], &done[i], &action[i]);
+      if (i < trace_n) {
+        size_t o = (size_t)k * trace_n + i;
+        tr_s[o] = s2;
+        tr_a[o] = action[i];
+        tr_r[o] = reward[i];
+        tr_d[o] = done[i];
+      }
+    }
+    if (shared)
+      for (size_t kk = 0; kk < K; ++kk) Q[kk] = Q[kk] + sum[kk];
+  }
+  free(tab);
+  free(sum);
+  return 0;
+}
+
+/* orc_run for per-env tables restricted to envs [lo, hi), env-major: lets the
+ * timing harness spread envs over host threads (envs are independent, and the
+ * draws are keyed by the global env index, so the results are orc_run's). */
+int orc_run_range(const orc_config* c, int32_t lo, int32_t hi, const uint8_t* cls,
+                  const float* cr, const int32_t* start, float* Q, int32_t* s,
+                  int32_t* ep_step, int32_t* episode, float* reward, uint8_t* done,
+                  uint8_t* action, uint64_t t0, int32_t n_steps) {
+  if (c->table_mode == 1) return -1;
+  const int A = c->n_actions;
+  const size_t S = (size_t)c->width * c->height;
+  const size_t K = S * A;
+  int cap = eps_cap(c);
+  float* tab = (float*)malloc((size_t)cap * sizeof(float));
+  if (!tab) return -3;
+  int len = orc_eps_table(c, tab, cap);
+  for (int i = lo; i < hi; ++i) {
+    size_t mo = c->map_mode == 1 ? 0 : (size_t)i * S;
+    for (int k = 0; k < n_steps; ++k) {
+      uint64_t t = t0 + (uint64_t)k;
+      float u;
+      int32_t ar;
+      orc_explore_draw(c->seed, (uint32_t)i, t, A, &u, &ar);
+      float eps = eps_at(c, tab, len, t, episode[i]);
+      env_step(c, eps, u, ar, cls + mo, cr ? cr + mo : NULL, Q + (size_t)i * K, NULL, start[i],
+               &s[i], &ep_step[i], &episode[i], &reward[i], &done[i], &action[i]);
+    }
+  }
+  free(tab);
+  return 0;
+}

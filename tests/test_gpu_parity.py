@@ -1,0 +1,274 @@
+"""GPU parity: the HIP engine, called through its C ABI, against the CPU oracle on
+the same seeded inputs.  Bar: trajectories (s', action, reward, done) bit-exact;
+fp32 Q-tables within 1e-5 relative (the tests assert the stronger bit equality
+first and report the relative error if that fails)."""
+import numpy as np
+import pytest
+
+pytestmark = pytest.mark.gpu
+
+REL_TOL = 1e-5  # BASELINE north_star: fp32 Q-tables within 1e-5 relative
+
+
+def assert_q_close(got, want):
+    if np.array_equal(got, want):
+        return
+    denom = np.maximum(np.maximum(np.abs(got), np.abs(want)), 1e-30)
+    rel = np.abs(got - want) / denom
+    assert rel.max() <= REL_TOL, "Q tables differ: max rel %.3g at %s" % (rel.max(), np.argmax(rel))
+    pytest.fail("Q tables within 1e-5 but not bit-identical (max rel %.3g)" % rel.max())
+
+
+def assert_trace_equal(got, want):
+    for k in ("s_next", "action", "reward", "done"):
+        if not np.array_equal(got[k], want[k]):
+            bad = np.argwhere(got[k] != want[k])[0]
+            pytest.fail("trace %s differs first at step %d env %d: %r vs %r"
+                        % (k, bad[0], bad[1], got[k][tuple(bad)], want[k][tuple(bad)]))
+
+
+def run_both(gpu, oracle, cfg, cls, start, n_steps, cr=None, chunks=None, trace_n=None, stream=None):
+    N = cfg.n_envs
+    trace_n = N if trace_n is None else trace_n
+    A, S = cfg.n_actions, cfg.width * cfg.height
+    n_tables = 1 if cfg.table_mode == gpu.TABLE_SHARED else N
+    with gpu.Engine(cfg, 0) as eng:
+        eng.set_maps(cls, start, cr)
+        eng.set_trace(trace_n, n_steps)
+        if stream is not None:
+            eng.set_exploration_stream(*stream)
+        for c in (chunks or [n_steps]):
+            eng.run_fused(c)
+        tr = eng.get_trace(n_steps)
+        q = eng.q_get(0, n_tables).reshape(n_tables, S, A)
+        st = eng.get_state()
+        assert eng.step_count == n_steps
+    Q = np.zeros((n_tables, S, A), np.float32)
+    ost = oracle.new_state(cfg, start)
+    want = oracle.run(cfg, cls, cr, start, Q, ost, 0, n_steps, trace_n=trace_n,
+                      u=None if stream is None else stream[0], a_rand=None if stream is None else stream[1])
+    assert_trace_equal(tr, want)
+    for k in ("s", "ep_step", "episode", "reward", "done", "action"):
+        assert np.array_equal(st[k], ost[k]), k
+    assert_q_close(q, Q)
+    return tr, q
+
+
+# ---- per-env tables, fused ------------------------------------------------------
+
+@pytest.mark.parametrize("N,W,H,T,steps", [
+    (1, 10, 10, 0, 300),       # one env, no time limit
+    (65, 7, 5, 11, 200),       # ragged: not a multiple of the wave or of 16 cells
+    (512, 32, 32, 256, 1000),  # config 2 shape, reduced N
+    (4096, 16, 16, 128, 300),  # config 4 shape, reduced N
+])
+def test_fused_per_env_matches_oracle(gpu, oracle, N, W, H, T, steps):
+    cls, start = gpu.gen_maps_bernoulli(7, N, N, W, H, 0.15, 0.03)
+    cfg = gpu.make_config(N, W, H, episode_len=T, eps0=0.1, gamma=0.95, seed=11, trap_reward=-1.0)
+    tr, _ = run_both(gpu, oracle, cfg, cls, start, steps)
+    if N >= 512:
+        assert tr["done"].sum() > 0  # goals reached: the restart path ran
+
+
+def test_fused_chunked_equals_one_launch(gpu, oracle):
+    """K steps in one launch == the same steps split over launches (odd splits
+    exercise the two-steps-per-Philox-block bookkeeping)."""
+    N, W, H = 300, 12, 9
+    cls, start = gpu.gen_maps_bernoulli(3, N, N, W, H, 0.2)
+    cfg = gpu.make_config(N, W, H, episode_len=20, eps0=0.3, seed=5)
+    run_both(gpu, oracle, cfg, cls, start, 101, chunks=[1, 1, 3, 7, 30, 59])
+
+
+def test_fused_large_map_global_path(gpu, oracle):
+    """Maps too large for LDS are read from global memory (config 5 shape: 8
+    actions, value-noise walls, per-cell rewards, linear epsilon)."""
+    N, W, H = 6, 256, 256
+    cls, start, cr = gpu.gen_maps_noise(21, N, W, H, 16, 0.25, 0.05, 10.0)
+    cfg = gpu.make_config(N, W, H, n_actions=8, episode_len=64, eps_mode=gpu.EPS_EPISODE_LINEAR, eps0=1.0,
+                          eps_end=0.05, eps_span=10, seed=2,
+                          reward_flags=gpu.REWARD_CELLS | gpu.REWARD_BASE_CELLS)
+    assert (cls == 3).sum(axis=1).tolist() == [W * H // 4] * N
+    tr, _ = run_both(gpu, oracle, cfg, cls, start, 1500, cr=cr)
+    assert len(np.unique(tr["action"])) == 8
+
+
+def test_fused_shared_map_per_env_tables(gpu, oracle):
+    N, W, H = 200, 20, 20
+    cls, start = gpu.gen_maps_bernoulli(4, 1, N, W, H, 0.15)
+    cfg = gpu.make_config(N, W, H, map_mode=gpu.MAP_SHARED, episode_len=50, eps0=0.2, seed=8)
+    run_both(gpu, oracle, cfg, cls, start, 400)
+
+
+def test_fused_supplied_exploration_stream(gpu, oracle):
+    """'The same supplied exploration random stream': numpy draws replace Philox."""
+    N, W, H, T = 128, 8, 8, 150
+    cls, start = gpu.gen_maps_bernoulli(9, N, N, W, H, 0.1)
+    cfg = gpu.make_config(N, W, H, episode_len=30, eps0=0.25, seed=1)
+    rng = np.random.default_rng(0)
+    u = rng.random((T, N), dtype=np.float32)
+    a = rng.integers(0, 4, (T, N)).astype(np.int32)
+    run_both(gpu, oracle, cfg, cls, start, T, stream=(u, a))
+
+
+@pytest.mark.parametrize("eps_mode", ["step", "episode"])
+def test_fused_eps_schedules_and_zero_floor(gpu, oracle, eps_mode):
+    N, W, H = 100, 10, 10
+    cls, start = gpu.gen_maps_bernoulli(5, N, N, W, H, 0.1)
+    kw = (dict(eps_mode=gpu.EPS_STEP_MULT, eps_span=400) if eps_mode == "step"
+          else dict(eps_mode=gpu.EPS_EPISODE_MULT, eps_span=50))
+    cfg = gpu.make_config(N, W, H, episode_len=25, eps0=1.0, eps_decay=0.99, seed=4,
+                          max_mode=gpu.MAX_ZERO_FLOOR, **kw)
+    run_both(gpu, oracle, cfg, cls, start, 500)
+
+
+def test_fused_sticky_done_without_auto_reset(gpu, oracle):
+    """auto_reset = 0: done stays set and stepping goes on (src/environment.cu:44-46)."""
+    N, W, H = 64, 5, 5
+    cls = np.zeros((N, W * H), np.uint8)
+    cls[:, W - 1] = 1
+    start = np.full(N, (H // 2) * W + W // 2, np.int32)
+    cfg = gpu.make_config(N, W, H, auto_reset=0, goal_mode=gpu.GOAL_ON_RESULT, eps0=1.0, seed=6)
+    tr, _ = run_both(gpu, oracle, cfg, cls, start, 200)
+    d = tr["done"]
+    assert d[-1].sum() > 0 and (np.diff(d.astype(int), axis=0) >= 0).all()
+
+
+# ---- the decomposed calls equal the fused kernel --------------------------------
+
+@pytest.mark.parametrize("shared", [False, True])
+def test_select_step_update_equals_fused(gpu, oracle, shared):
+    N, W, H, T = 333, 9, 9, 60
+    n_maps = 1 if shared else N
+    cls, start = gpu.gen_maps_bernoulli(12, n_maps, N, W, H, 0.15, 0.05)
+    cfg = gpu.make_config(N, W, H, episode_len=13, eps0=0.3, seed=3,
+                          table_mode=gpu.TABLE_SHARED if shared else gpu.TABLE_PER_ENV,
+                          map_mode=gpu.MAP_SHARED if shared else gpu.MAP_PER_ENV)
+    n_tables = 1 if shared else N
+    with gpu.Engine(cfg, 0) as a, gpu.Engine(cfg, 0) as b:
+        for e in (a, b):
+            e.set_maps(cls, start)
+            e.set_trace(N, T)
+        a.run_fused(T)
+        acts = []
+        for _ in range(T):
+            acts.append(b.select())
+            b.step()
+            b.update()
+        ta, tb = a.get_trace(T), b.get_trace(T)
+        assert_trace_equal(tb, ta)
+        assert np.array_equal(np.array(acts, np.uint8), ta["action"])
+        assert np.array_equal(a.q_get(0, n_tables), b.q_get(0, n_tables))
+        sa, sb = a.get_state(), b.get_state()
+        for k in sa:
+            assert np.array_equal(sa[k], sb[k]), k
+        assert a.step_count == b.step_count == T
+
+
+# ---- shared table: ordered reduction ----------------------------------------------
+
+@pytest.mark.parametrize("N,W,H,steps", [(64, 4, 4, 50), (5000, 16, 16, 120), (65536, 64, 64, 12)])
+def test_shared_table_matches_oracle(gpu, oracle, N, W, H, steps):
+    cls, start = gpu.gen_maps_bernoulli(2, 1, N, W, H, 0.15)
+    cfg = gpu.make_config(N, W, H, table_mode=gpu.TABLE_SHARED, map_mode=gpu.MAP_SHARED, lr=0.05,
+                          eps0=0.2, episode_len=0, seed=13)
+    run_both(gpu, oracle, cfg, cls, start, steps, trace_n=min(N, 4096))
+
+
+def test_shared_table_all_envs_on_one_cell(gpu, oracle):
+    """Degenerate segment: every env hits the same (s,a) keys."""
+    N, W, H = 3000, 3, 3
+    cls = np.zeros((1, W * H), np.uint8)
+    cls[0, 8] = 1
+    start = np.zeros(N, np.int32)
+    cfg = gpu.make_config(N, W, H, table_mode=gpu.TABLE_SHARED, map_mode=gpu.MAP_SHARED, lr=0.05,
+                          eps0=0.5, episode_len=6, seed=1)
+    run_both(gpu, oracle, cfg, cls, start, 40)
+
+
+def test_shared_table_run_to_run_identity(gpu):
+    N, W, H = 20000, 32, 32
+    cls, start = gpu.gen_maps_bernoulli(6, 1, N, W, H, 0.15)
+    cfg = gpu.make_config(N, W, H, table_mode=gpu.TABLE_SHARED, map_mode=gpu.MAP_SHARED, lr=0.05,
+                          eps0=0.2, seed=21)
+    qs = []
+    for _ in range(2):
+        with gpu.Engine(cfg, 0) as eng:
+            eng.set_maps(cls, start)
+            eng.run_fused(100)
+            qs.append(eng.q_get(0))
+    assert np.array_equal(qs[0], qs[1])
+    assert np.count_nonzero(qs[0]) > 100
+
+
+# ---- explicit batches (CudaQLearning::update_batch) --------------------------------
+
+@pytest.mark.parametrize("mode", [0, 1])
+@pytest.mark.parametrize("n", [1, 10, 1024, 5000])
+def test_td_update_batch_matches_oracle(gpu, oracle, mode, n):
+    W, H, A = 10, 10, 4
+    S = W * H
+    cfg = gpu.make_config(1, W, H, max_mode=mode, table_mode=gpu.TABLE_SHARED, map_mode=gpu.MAP_SHARED)
+    rng = np.random.default_rng(n + mode)
+    Q0 = rng.normal(0, 1, (S, A)).astype(np.float32)
+    s, a, s2 = rng.integers(0, S, n), rng.integers(0, A, n), rng.integers(0, S, n)
+    r = rng.normal(0, 1, n).astype(np.float32)
+    done = (rng.random(n) < 0.2).astype(np.uint8)
+    with gpu.Engine(cfg, 0) as eng:
+        eng.q_set(0, Q0)
+        eng.td_update(0, s, a, r, s2, done)
+        got = eng.q_get(0)
+    want = Q0.copy().reshape(-1)
+    oracle.td_update_batch(want, S, A, s, a, r, s2, done, 0.1, 0.99, mode)
+    assert_q_close(got.reshape(-1), want)
+
+
+# ---- step rule, exhaustively, through the engine ------------------------------------
+
+def test_step_rule_brute_force_against_float_grid(gpu, oracle):
+    """Every (cell, action) on float grids holding every class and threshold
+    edge value: engine step on the classified grid == src/kernels.cu:13-66."""
+    from test_oracle_pins import EDGE_VALUES
+    W, H = 5, 4
+    S = W * H
+    vals = np.array(EDGE_VALUES, np.float32)
+    rng = np.random.default_rng(3)
+    actions = list(range(-1, 6))
+    for trial in range(4):
+        grid = vals[rng.integers(0, len(vals), S)].astype(np.float32)
+        cls, cr = gpu.classify_grid(grid)
+        N = S * len(actions)
+        cfg = gpu.make_config(N, W, H, map_mode=gpu.MAP_SHARED, auto_reset=0, reward_flags=gpu.REWARD_CELLS)
+        start = np.repeat(np.arange(S, dtype=np.int32), len(actions))
+        act = np.tile(np.array(actions, np.int32), S)
+        with gpu.Engine(cfg, 0) as eng:
+            eng.set_maps(cls, start, cr)
+            eng.step(act)
+            st = eng.get_state()
+        for i in range(N):
+            x, y, r, d = oracle.step_e2(grid, W, H, int(start[i]) % W, int(start[i]) // W, 0, int(act[i]))
+            assert (st["s"][i], st["reward"][i], st["done"][i]) == (y * W + x, np.float32(r), d), (trial, i)
+
+
+def test_full_size_properties_config4_slice(gpu):
+    """Size-independent properties at a large N (no oracle): positions stay on
+    non-blocking cells, rewards come from the rule's value set, every table
+    entry of a never-visited (walled) cell stays zero, and two runs agree."""
+    N, W, H, steps = 1 << 17, 16, 16, 256
+    cls, start = gpu.gen_maps_bernoulli(0, N, N, W, H, 0.1, 0.02)
+    cfg = gpu.make_config(N, W, H, episode_len=128, eps0=0.1, gamma=0.95, seed=0, trap_reward=-1.0)
+    outs = []
+    for _ in range(2):
+        with gpu.Engine(cfg, 0) as eng:
+            eng.set_maps(cls, start)
+            eng.run_fused(steps)
+            st = eng.get_state()
+            q = eng.q_get(0, 2048)
+        outs.append((st, q))
+    st, q = outs[0]
+    assert all(np.array_equal(outs[0][0][k], outs[1][0][k]) for k in st) and np.array_equal(q, outs[1][1])
+    here = cls[np.arange(N), st["s"]]
+    assert (here < 2).all()
+    assert set(np.unique(st["reward"]).tolist()) <= {np.float32(-0.01), np.float32(1.0), np.float32(-1.0)}
+    blocked = cls[:2048] >= 2
+    assert (q[blocked] == 0).all()
+    assert (st["ep_step"] < 128).all() and st["episode"].min() >= 2
