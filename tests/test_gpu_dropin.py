@@ -1,0 +1,231 @@
+"""The reference-shaped host classes (Environment, EnvironmentBridge,
+CudaQLearning, module cudarl_core) on the HIP engine.  The first block restates
+tests/test_environment.cpp case by case; the rest covers what the reference
+leaves untested (bridge tuple shape, update_batch, error messages)."""
+import json
+import os
+import sys
+
+import numpy as np
+import pytest
+
+pytestmark = pytest.mark.gpu
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+LIBDIR = os.path.join(ROOT, "cudarl-arena_amd", "lib")
+
+
+@pytest.fixture(scope="module")
+def core(gpu):
+    sys.path.insert(0, LIBDIR)
+    import cudarl_core
+    return cudarl_core
+
+
+def approx(v):
+    return pytest.approx(v, rel=1e-6)
+
+
+# ---- tests/test_environment.cpp ---------------------------------------------------
+
+def test_environment_initialization(core):  # cpp:5-27
+    env = core.RawEnvironment(0)
+    assert (env.getWidth(), env.getHeight()) == (10, 10)
+    assert (env.getAgentX(), env.getAgentY()) == (5, 5)
+    assert env.getReward() == 0.0
+    assert env.isDone() is False
+
+
+def test_environment_reset(core):  # cpp:29-51
+    env = core.RawEnvironment(0)
+    env.step(1)
+    env.step(1)
+    env.reset()
+    assert (env.getAgentX(), env.getAgentY()) == (5, 5)
+    assert env.getReward() == 0.0
+    assert env.isDone() is False
+
+
+def test_environment_step(core):  # cpp:53-98
+    for action, want in ((1, (6, 5)), (2, (5, 6)), (3, (4, 5)), (0, (5, 4))):
+        env = core.RawEnvironment(0)
+        env.step(action)
+        assert (env.getAgentX(), env.getAgentY()) == want
+    small = core.RawEnvironment(1, 3, 3)
+    small.step(1)
+    assert small.getAgentX() == 2
+    small.step(1)
+    assert small.getAgentX() == 2
+    env = core.RawEnvironment(0)
+    env.step(1)
+    assert env.getReward() == approx(-0.01)
+
+
+def test_environment_goal_detection(core):  # cpp:100-120
+    env = core.RawEnvironment(0, 5, 5)
+    env.reset()
+    for a in (1, 1, 0, 0):
+        env.step(a)
+    assert env.isDone() is True
+    assert env.getReward() == approx(1.0)
+
+
+def test_environment_grid_access(core):  # cpp:122-139
+    env = core.RawEnvironment(0, 5, 5)
+    grid = env.getGrid()
+    assert len(grid) == 25
+    assert env.getCellValue(4, 0) == approx(1.0)
+    assert env.getCellValue(10, 10) == 0.0
+    others = np.delete(np.array(grid), 4)
+    assert (others >= 0).all() and (others <= 0.5).all()  # src/environment.cu:142
+
+
+def test_golden_catch2_cases_through_the_engine(core):
+    g = json.load(open(os.path.join(ROOT, "tests", "golden", "catch2_environment.json")))
+    for case in g["cases"]:
+        env = core.RawEnvironment(0, case["width"], case["height"])
+        for a in case.get("actions", []):
+            env.step(a)
+        if case.get("reset_after"):
+            env.reset()
+        e = case["expect"]
+        got = dict(x=env.getAgentX(), y=env.getAgentY(), reward=env.getReward(), done=env.isDone())
+        for k, v in e.items():
+            assert got[k] == (approx(v) if k == "reward" else v), case["name"]
+
+
+def test_done_is_sticky_and_invalid_action_stays(core):  # src/environment.cu:17-48
+    env = core.RawEnvironment(0, 5, 5)
+    for a in (1, 1, 0, 0):
+        env.step(a)
+    env.step(3)  # walk off the goal: done stays
+    assert env.isDone() and (env.getAgentX(), env.getAgentY()) == (3, 0)
+    assert env.getReward() == approx(-0.01)
+    env.step(7)  # no such action: no move
+    assert (env.getAgentX(), env.getAgentY()) == (3, 0)
+    env.reset()
+    assert not env.isDone()
+
+
+# ---- EnvironmentBridge / cudarl_core.Environment ----------------------------------
+
+def test_bridge_surface(core):  # src/environment_bridge.cu, src/python_bindings.cpp:8-26
+    assert core.__version__ == "0.1.0"
+    env = core.Environment()
+    assert (env.get_width(), env.get_height()) == (10, 10)
+    env = core.Environment(width=6, height=4)
+    obs = env.reset()
+    assert isinstance(obs, list) and len(obs) == 24
+    assert env.get_agent_position() == (3, 2)
+    obs2, reward, done, info = env.step(1)
+    assert obs2 == obs and obs2 == env.get_observation()  # the grid is static
+    assert reward == approx(-0.01) and done is False
+    assert info == "agent_pos: (4,2)"  # src/environment_bridge.cu:30-31
+    for name in ("reset", "step", "get_observation", "get_width", "get_height", "get_agent_position",
+                 "add_obstacle", "set_goal", "add_trap"):
+        assert hasattr(env, name)
+
+
+def test_bridge_obstacle_goal_trap_take_effect(core, oracle):
+    """Upstream these three only print; here they edit the map, with the cell
+    semantics of src/kernels.cu:13-66 (checked against the float-grid oracle)."""
+    W = H = 5
+    env = core.Environment(W, H)
+    env.add_obstacle(3, 2)
+    env.add_trap(2, 1, -0.5)
+    env.add_trap(1, 2)  # default penalty -1.0 is still a trap here
+    env.set_goal(2, 4)
+    grid = np.array(env.get_observation(), np.float32)
+    assert grid[2 * W + 3] == -1.0 and grid[1 * W + 2] == -0.5 and grid[4 * W + 2] == 1.0
+    env.reset()
+    _, r, d, info = env.step(1)  # wall to the right
+    assert (r, d, info) == (approx(-0.01), False, "agent_pos: (2,2)")
+    _, r, d, info = env.step(0)  # trap above: penalty, no move
+    assert (r, d, info) == (approx(-0.5), False, "agent_pos: (2,2)")
+    _, r, d, info = env.step(3)  # default trap to the left
+    assert (r, d, info) == (approx(-1.0), False, "agent_pos: (2,2)")
+    _, r, d, info = env.step(2)
+    assert (r, d, info) == (approx(-0.01), False, "agent_pos: (2,3)")
+    _, r, d, info = env.step(2)  # the new goal
+    assert (r, d, info) == (approx(1.0), True, "agent_pos: (2,4)")
+    # wall and -0.5 trap agree with the reference's float rule
+    x, y, r, d = oracle.step_e2(grid, W, H, 2, 2, 0, 0)
+    assert (x, y, d) == (2, 2, 0) and r == np.float32(-0.5)
+
+
+# ---- CudaQLearning ------------------------------------------------------------------
+
+def test_q_learning_demo_of_main_cu(core):  # src/main.cu:26-94
+    q = core.CudaQLearning(10, 10, 4, 0.1, 0.99)
+    assert q.get_q_table() == [0.0] * 400
+    states = [(5, 5), (6, 5), (6, 4)]
+    nexts = [(6, 5), (6, 4), (6, 3)]
+    q.update_batch(states, [1, 0, 0], [-0.01, -0.01, -0.01], nexts, [False, False, False])
+    for a in range(4):
+        assert q.get_q_value(0, 0, a) == 0.0  # (0,0) never visited (src/main.cu:92-94)
+    assert q.get_q_value(5, 5, 1) == np.float32(np.float32(0.1) * np.float32(-0.01))
+    assert q.get_best_action(0, 0) == 0  # all-zero row: lowest index
+    assert q.get_best_action(5, 5) == 0  # Q(5,5,1) < 0: action 0 wins
+
+
+@pytest.mark.parametrize("mode", [0, 1])
+def test_q_learning_update_batch_matches_oracle(core, oracle, mode):
+    W, H, A, n = 7, 6, 4, 1024
+    rng = np.random.default_rng(mode)
+    q = core.CudaQLearning(W, H, A, 0.1, 0.99, mode)
+    Q0 = rng.normal(0, 1, W * H * A).astype(np.float32)
+    q.set_q_table(Q0.tolist())
+    xs, ys, nx, ny = (rng.integers(0, W, n), rng.integers(0, H, n), rng.integers(0, W, n),
+                      rng.integers(0, H, n))
+    a = rng.integers(0, A, n)
+    r = rng.normal(0, 1, n).astype(np.float32)
+    d = rng.random(n) < 0.2
+    q.update_batch(list(zip(xs.tolist(), ys.tolist())), a.tolist(), r.tolist(),
+                   list(zip(nx.tolist(), ny.tolist())), d.tolist())
+    want = Q0.copy()
+    oracle.td_update_batch(want, W * H, A, ys * W + xs, a, r, ny * W + nx, d.astype(np.uint8), 0.1, 0.99, mode)
+    got = np.array(q.get_q_table(), np.float32)
+    assert np.array_equal(got, want)
+    best = int(np.argmax(want.reshape(-1, A)[3 * W + 2]))
+    assert q.get_best_action(2, 3) == best
+
+
+def test_q_learning_errors(core):  # src/q_learning.cu:117-124,181-183,192-194,212-214
+    q = core.CudaQLearning(4, 4, 4)
+    with pytest.raises(RuntimeError, match="Batch size exceeds maximum batch size"):
+        q.update_batch([(0, 0)] * 1025, [0] * 1025, [0.0] * 1025, [(0, 0)] * 1025, [False] * 1025)
+    with pytest.raises(RuntimeError, match="Inconsistent batch sizes"):
+        q.update_batch([(0, 0)], [0, 1], [0.0], [(0, 0)], [False])
+    with pytest.raises(RuntimeError, match="Invalid Q-table size"):
+        q.set_q_table([0.0] * 5)
+    with pytest.raises(RuntimeError, match="Invalid state"):
+        q.get_best_action(4, 0)
+    with pytest.raises(RuntimeError, match="Invalid state or action"):
+        q.get_q_value(0, 0, 4)
+    q.update_batch([], [], [], [], [])  # empty batch is a no-op
+    assert q.get_q_table() == [0.0] * 64
+
+
+def test_engine_argument_errors(gpu):
+    cfg = gpu.make_config(8, 4, 4)
+    with gpu.Engine(cfg, 0) as eng:
+        with pytest.raises(gpu.CrlError) as e:
+            eng.step(None)  # no select before
+        assert e.value.code == -4
+        with pytest.raises(gpu.CrlError):
+            eng.update()
+        with pytest.raises(gpu.CrlError) as e:
+            eng.reset(4, 8)
+        assert e.value.code == -5
+        with pytest.raises(gpu.CrlError):
+            eng.set_maps(np.full((8, 16), 9, np.uint8), np.zeros(8, np.int32))
+        with pytest.raises(gpu.CrlError):
+            eng.set_maps(np.zeros((8, 16), np.uint8), np.full(8, 16, np.int32))
+        with pytest.raises(gpu.CrlError):
+            eng.td_update(0, [99], [0], [0.0], [0], [0])
+        with pytest.raises(gpu.CrlError):
+            eng.q_get(8)
+        eng.run_fused(0)
+        assert eng.step_count == 0
+    with pytest.raises(gpu.CrlError):
+        gpu.Engine(cfg, 99)

@@ -11,8 +11,12 @@ REL_TOL = 1e-5  # BASELINE north_star: fp32 Q-tables within 1e-5 relative
 
 
 def assert_q_close(got, want):
-    if np.array_equal(got, want):
+    # summed deltas can overflow a shared table (the effective step size is lr
+    # times the number of envs on one (s,a)); NaNs must then sit in the same places
+    if np.array_equal(got, want, equal_nan=True):
         return
+    assert np.array_equal(np.isfinite(got), np.isfinite(want))
+    got, want = np.nan_to_num(got, posinf=0, neginf=0), np.nan_to_num(want, posinf=0, neginf=0)
     denom = np.maximum(np.maximum(np.abs(got), np.abs(want)), 1e-30)
     rel = np.abs(got - want) / denom
     assert rel.max() <= REL_TOL, "Q tables differ: max rel %.3g at %s" % (rel.max(), np.argmax(rel))
@@ -166,12 +170,16 @@ def test_select_step_update_equals_fused(gpu, oracle, shared):
 
 # ---- shared table: ordered reduction ----------------------------------------------
 
-@pytest.mark.parametrize("N,W,H,steps", [(64, 4, 4, 50), (5000, 16, 16, 120), (65536, 64, 64, 12)])
-def test_shared_table_matches_oracle(gpu, oracle, N, W, H, steps):
+@pytest.mark.parametrize("N,W,H,steps,lr", [(64, 4, 4, 50, 0.05), (5000, 16, 16, 120, 0.002),
+                                            (5000, 16, 16, 120, 0.05),  # overflows: inf/nan parity
+                                            (65536, 64, 64, 12, 0.05)])
+def test_shared_table_matches_oracle(gpu, oracle, N, W, H, steps, lr):
     cls, start = gpu.gen_maps_bernoulli(2, 1, N, W, H, 0.15)
-    cfg = gpu.make_config(N, W, H, table_mode=gpu.TABLE_SHARED, map_mode=gpu.MAP_SHARED, lr=0.05,
+    cfg = gpu.make_config(N, W, H, table_mode=gpu.TABLE_SHARED, map_mode=gpu.MAP_SHARED, lr=lr,
                           eps0=0.2, episode_len=0, seed=13)
-    run_both(gpu, oracle, cfg, cls, start, steps, trace_n=min(N, 4096))
+    _, q = run_both(gpu, oracle, cfg, cls, start, steps, trace_n=min(N, 4096))
+    if lr < 0.01:
+        assert np.isfinite(q).all() and np.count_nonzero(q) > 50
 
 
 def test_shared_table_all_envs_on_one_cell(gpu, oracle):
