@@ -789,4 +789,20 @@ int crl_fused_kernel_info(crl_engine* e, char* name, size_t name_len, int32_t* g
   return CRL_OK;
 }
 
+int crl_probe_copy(size_t n_bytes, int repeats) {
+  if (n_bytes == 0 || n_bytes % 16 != 0 || repeats < 1) return fail(CRL_E_ARG, "n_bytes must be a positive multiple of 16");
+  DevBuf<uint8_t> src, dst;
+  if (src.alloc(n_bytes) != hipSuccess || dst.alloc(n_bytes) != hipSuccess)
+    return fail(CRL_E_ALLOC, "probe allocation failed");
+  HIP_TRY(hipMemset(src.p, 1, n_bytes));
+  HIP_TRY(hipMemset(dst.p, 0, n_bytes));
+  const size_t n16 = n_bytes / 16;
+  for (int i = 0; i < repeats; ++i)
+    hipLaunchKernelGGL(crl::k_probe_copy, dim3(256 * 16), dim3(256), 0, nullptr,
+                       reinterpret_cast<const uint4*>(src.p), reinterpret_cast<uint4*>(dst.p), n16);
+  HIP_TRY(hipGetLastError());
+  HIP_TRY(hipDeviceSynchronize());
+  return CRL_OK;
+}
+
 }  // extern "C"

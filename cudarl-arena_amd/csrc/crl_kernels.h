@@ -455,4 +455,12 @@ __global__ __launch_bounds__(kReduceBlock) void k_reduce_apply(float* __restrict
   if (wave == 0 && k < K) Q[k] = Q[k] + acc;
 }
 
+// plain copy of n16 16-byte words: the known-size launch that calibrates the
+// hardware traffic counters
+__global__ __launch_bounds__(256) void k_probe_copy(const uint4* __restrict__ src,
+                                                     uint4* __restrict__ dst, const size_t n16) {
+  const size_t stride = (size_t)gridDim.x * blockDim.x;
+  for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < n16; i += stride) dst[i] = src[i];
+}
+
 }  // namespace crl

@@ -83,7 +83,7 @@ EXPORTS = [
     "crl_set_state", "crl_get_step_count", "crl_set_step_count", "crl_q_get", "crl_q_set",
     "crl_q_get_range", "crl_set_trace", "crl_get_trace", "crl_set_exploration_stream",
     "crl_device_ptr", "crl_fused_kernel_info", "crl_philox4x32_10", "crl_explore_draw",
-    "crl_eps_table", "crl_gen_maps_bernoulli", "crl_gen_maps_noise",
+    "crl_eps_table", "crl_gen_maps_bernoulli", "crl_gen_maps_noise", "crl_probe_copy",
 ]
 
 
@@ -132,6 +132,7 @@ def load():
     lib.crl_eps_table.argtypes = [C.POINTER(Config), vp, i32, C.POINTER(i32)]
     lib.crl_gen_maps_bernoulli.argtypes = [u64, i32, i32, i32, i32, f32, f32, vp, vp]
     lib.crl_gen_maps_noise.argtypes = [u64, i32, i32, i32, i32, f32, f32, f32, vp, vp, vp]
+    lib.crl_probe_copy.argtypes = [C.c_size_t, C.c_int]
     _lib = lib
     return lib
 

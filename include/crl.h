@@ -215,6 +215,11 @@ int crl_device_ptr(crl_engine* e, int32_t which, void** out);
 int crl_fused_kernel_info(crl_engine* e, char* name, size_t name_len, int32_t* grid,
                           int32_t* block, int32_t* lds_bytes);
 
+/* Measurement helper (no reference counterpart): one launch of a plain copy
+ * kernel `k_probe_copy` moving n_bytes from one device buffer to another, so
+ * that hardware traffic counters can be scaled by a launch of known size. */
+int crl_probe_copy(size_t n_bytes, int repeats);
+
 /* -- host-side helpers (no device needed) ----------------------------------- */
 
 /* Philox4x32-10 (Salmon et al. 2011), exposed for tests. */

@@ -196,7 +196,7 @@ def test_shared_table_all_envs_on_one_cell(gpu, oracle):
 def test_shared_table_run_to_run_identity(gpu):
     N, W, H = 20000, 32, 32
     cls, start = gpu.gen_maps_bernoulli(6, 1, N, W, H, 0.15)
-    cfg = gpu.make_config(N, W, H, table_mode=gpu.TABLE_SHARED, map_mode=gpu.MAP_SHARED, lr=0.05,
+    cfg = gpu.make_config(N, W, H, table_mode=gpu.TABLE_SHARED, map_mode=gpu.MAP_SHARED, lr=0.004,
                           eps0=0.2, seed=21)
     qs = []
     for _ in range(2):
@@ -204,7 +204,7 @@ def test_shared_table_run_to_run_identity(gpu):
             eng.set_maps(cls, start)
             eng.run_fused(100)
             qs.append(eng.q_get(0))
-    assert np.array_equal(qs[0], qs[1])
+    assert np.isfinite(qs[0]).all() and np.array_equal(qs[0], qs[1])
     assert np.count_nonzero(qs[0]) > 100
 
 
