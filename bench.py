@@ -95,7 +95,7 @@ class HipEvents:
         return float(ms.value)
 
 
-def time_gpu(key, steps, warmup, launches=1, n_override=None):
+def time_gpu(key, steps, warmup, launches=1, n_override=None, resident=0):
     """-> dict(steps_per_s, ms_per_step, kernel_ms, wall_s, info)"""
     wl = WORKLOADS[key]
     cfg, cls, start, cr = build_workload(key, n_override)
@@ -104,6 +104,8 @@ def time_gpu(key, steps, warmup, launches=1, n_override=None):
     with pycrl.Engine(cfg, 0) as eng:
         eng.set_maps(cls, start, cr)
         del cls, cr
+        if resident:
+            eng.set_resident_envs(resident)
         info = eng.fused_kernel_info()
         if warmup:
             eng.run_fused(warmup)
@@ -173,6 +175,7 @@ def main():
     ap.add_argument("--workload", default="c4", choices=sorted(WORKLOADS))
     ap.add_argument("--launches", type=int, default=1, help="split the K timed steps over this many launches")
     ap.add_argument("--envs", type=int, default=None, help="override the env count (not a headline figure)")
+    ap.add_argument("--resident", type=int, default=0, help="envs in flight at once (0 = automatic)")
     ap.add_argument("--probe-copy", type=int, default=0, metavar="MIB",
                     help="only run one plain copy kernel of this many MiB (calibrates rocprofv3 counters)")
     ap.add_argument("--no-cpu", action="store_true", help="skip the cpu_baseline leg")
@@ -193,7 +196,7 @@ def main():
     wl = WORKLOADS[key]
     steps = args.steps if args.steps is not None else wl["steps"]
     warmup = args.warmup if args.warmup is not None else wl["warmup"]
-    g = time_gpu(key, steps, warmup, args.launches, args.envs)
+    g = time_gpu(key, steps, warmup, args.launches, args.envs, args.resident)
 
     achieved = g["steps_per_s"] * wl["bytes"] / 1e9
     # the dominant kernel's own duration (device events around its launches)

@@ -83,60 +83,100 @@ __device__ __forceinline__ void step_rule(const Rules& R, ClassOf cls, const flo
   reward = r;
 }
 
+// One table row in registers.  Named scalars passed BY VALUE: an element picked
+// by a run-time action index must compile to a chain of selects.  Through a
+// reference the optimiser folds "select of two loads" into one indexed load
+// and the row ends up in scratch memory.
 template <int A>
-struct Row {
-  float v[A];
+struct Row;
+
+template <>
+struct Row<4> {
+  float q0, q1, q2, q3;
+};
+template <>
+struct Row<8> {
+  float q0, q1, q2, q3, q4, q5, q6, q7;
 };
 
-template <int A>
-__device__ __forceinline__ Row<A> load_row(const float* __restrict__ p) {
-  Row<A> r;
-  const float4* p4 = reinterpret_cast<const float4*>(p);
-#pragma unroll
-  for (int i = 0; i < A / 4; ++i) {
-    const float4 t = p4[i];
-    r.v[4 * i + 0] = t.x;
-    r.v[4 * i + 1] = t.y;
-    r.v[4 * i + 2] = t.z;
-    r.v[4 * i + 3] = t.w;
-  }
-  return r;
+__device__ __forceinline__ Row<4> load_row4(const float* __restrict__ p) {
+  const float4 t = *reinterpret_cast<const float4*>(p);
+  return Row<4>{t.x, t.y, t.z, t.w};
 }
+__device__ __forceinline__ Row<8> load_row8(const float* __restrict__ p) {
+  const float4 t = reinterpret_cast<const float4*>(p)[0];
+  const float4 u = reinterpret_cast<const float4*>(p)[1];
+  return Row<8>{t.x, t.y, t.z, t.w, u.x, u.y, u.z, u.w};
+}
+template <int A>
+__device__ __forceinline__ Row<A> load_row(const float* __restrict__ p);
+template <>
+__device__ __forceinline__ Row<4> load_row<4>(const float* __restrict__ p) { return load_row4(p); }
+template <>
+__device__ __forceinline__ Row<8> load_row<8>(const float* __restrict__ p) { return load_row8(p); }
 
 // lowest index wins ties (src/q_learning.cu:200-206: strict >)
-template <int A>
-__device__ __forceinline__ int row_argmax(const Row<A>& r) {
-  int best = 0;
-  float bv = r.v[0];
-#pragma unroll
-  for (int a = 1; a < A; ++a) {
-    const bool gt = r.v[a] > bv;
-    bv = gt ? r.v[a] : bv;
-    best = gt ? a : best;
-  }
-  return best;
+__device__ __forceinline__ void amax_step(float v, int i, float& bv, int& bi) {
+  const bool gt = v > bv;
+  bv = gt ? v : bv;
+  bi = gt ? i : bi;
+}
+__device__ __forceinline__ int row_argmax(const Row<4> r) {
+  float bv = r.q0;
+  int bi = 0;
+  amax_step(r.q1, 1, bv, bi);
+  amax_step(r.q2, 2, bv, bi);
+  amax_step(r.q3, 3, bv, bi);
+  return bi;
+}
+__device__ __forceinline__ int row_argmax(const Row<8> r) {
+  float bv = r.q0;
+  int bi = 0;
+  amax_step(r.q1, 1, bv, bi);
+  amax_step(r.q2, 2, bv, bi);
+  amax_step(r.q3, 3, bv, bi);
+  amax_step(r.q4, 4, bv, bi);
+  amax_step(r.q5, 5, bv, bi);
+  amax_step(r.q6, 6, bv, bi);
+  amax_step(r.q7, 7, bv, bi);
+  return bi;
 }
 
-template <int A>
-__device__ __forceinline__ float row_get(const Row<A>& r, int a) {
-  float q = r.v[0];
-#pragma unroll
-  for (int i = 1; i < A; ++i) q = (a == i) ? r.v[i] : q;
+__device__ __forceinline__ float row_get(const Row<4> r, int a) {
+  float q = r.q0;
+  q = (a == 1) ? r.q1 : q;
+  q = (a == 2) ? r.q2 : q;
+  q = (a == 3) ? r.q3 : q;
+  return q;
+}
+__device__ __forceinline__ float row_get(const Row<8> r, int a) {
+  float q = r.q0;
+  q = (a == 1) ? r.q1 : q;
+  q = (a == 2) ? r.q2 : q;
+  q = (a == 3) ? r.q3 : q;
+  q = (a == 4) ? r.q4 : q;
+  q = (a == 5) ? r.q5 : q;
+  q = (a == 6) ? r.q6 : q;
+  q = (a == 7) ? r.q7 : q;
   return q;
 }
 
-template <int A>
-__device__ __forceinline__ void row_set(Row<A>& r, int a, float q) {
-#pragma unroll
-  for (int i = 0; i < A; ++i) r.v[i] = (a == i) ? q : r.v[i];
+__device__ __forceinline__ Row<4> row_set(const Row<4> r, int a, float q) {
+  return Row<4>{(a == 0) ? q : r.q0, (a == 1) ? q : r.q1, (a == 2) ? q : r.q2, (a == 3) ? q : r.q3};
+}
+__device__ __forceinline__ Row<8> row_set(const Row<8> r, int a, float q) {
+  return Row<8>{(a == 0) ? q : r.q0, (a == 1) ? q : r.q1, (a == 2) ? q : r.q2, (a == 3) ? q : r.q3,
+                (a == 4) ? q : r.q4, (a == 5) ? q : r.q5, (a == 6) ? q : r.q6, (a == 7) ? q : r.q7};
 }
 
 // max_a' Q[s',a'] (src/gpu/kernels.cu:35-45), or floored at 0 (src/kernels.cu:101-110)
-template <int A>
-__device__ __forceinline__ float row_max(const Row<A>& r, bool done, int max_mode) {
-  float m = r.v[0];
-#pragma unroll
-  for (int a = 1; a < A; ++a) m = fmaxf(m, r.v[a]);
+__device__ __forceinline__ float row_max(const Row<4> r, bool done, int max_mode) {
+  float m = fmaxf(fmaxf(r.q0, r.q1), fmaxf(r.q2, r.q3));
+  if (max_mode == 1) m = fmaxf(0.0f, m);
+  return done ? 0.0f : m;
+}
+__device__ __forceinline__ float row_max(const Row<8> r, bool done, int max_mode) {
+  float m = fmaxf(fmaxf(fmaxf(r.q0, r.q1), fmaxf(r.q2, r.q3)), fmaxf(fmaxf(r.q4, r.q5), fmaxf(r.q6, r.q7)));
   if (max_mode == 1) m = fmaxf(0.0f, m);
   return done ? 0.0f : m;
 }

@@ -5,6 +5,8 @@
 
 #include <cstdarg>
 #include <cstdio>
+#include <algorithm>
+#include <cstdlib>
 #include <cstring>
 #include <new>
 #include <string>
@@ -70,6 +72,7 @@ struct crl_engine {
   size_t S = 0, K = 0;
   int n_maps = 0, n_tables = 0, map_words = 0;
   uint64_t t = 0;
+  long resident_envs = 0;  // 0 = automatic
 
   DevBuf<int32_t> s, ep_step, episode, start, act;
   DevBuf<float> reward;
@@ -84,9 +87,13 @@ struct crl_engine {
   DevBuf<float> tr_r;
   DevBuf<uint8_t> tr_done;
   bool have_transition = false, have_actions = false;
-  // (key, delta) scratch of the ordered reduction
+  // (key, delta) scratch of the ordered reduction, and the block sums its
+  // first pass hands to the key owners
   DevBuf<int32_t> key;
   DevBuf<float> delta;
+  DevBuf<uint2> handoff;
+  DevBuf<uint8_t> handoff_count;
+  bool lds_opt_in = false;
   // scratch of crl_td_update
   DevBuf<int32_t> b_s, b_a, b_s2;
   DevBuf<float> b_r;
@@ -171,6 +178,8 @@ struct crl_engine {
 namespace {
 
 constexpr int kLdsMapLimitBytes = 64 * 1024;
+constexpr size_t kLastLevelCacheBytes = (size_t)256 << 20;  // MI355X Infinity Cache
+constexpr long kLanesOneWavePerSimd = 256L * 4 * 64;        // 256 CUs x 4 SIMDs x 64 lanes
 
 // launch geometry of the fused per-env kernel
 struct FusedPlan {
@@ -201,6 +210,18 @@ FusedPlan plan_fused(const crl_engine* e) {
     }
   }
   p.grid = (e->N + p.block - 1) / p.block;
+  // Envs live on the chip at once.  A block works through its chunks one after
+  // the other, so a smaller grid means fewer tables in flight: when all tables
+  // together exceed the last-level cache, keep as many in flight as fit into
+  // it (but never less than one wave per SIMD of the whole chip).
+  long resident = e->resident_envs;
+  if (resident <= 0) {
+    const size_t table_bytes = e->K * sizeof(float);
+    resident = e->N;
+    if ((size_t)e->N * table_bytes > kLastLevelCacheBytes)
+      resident = std::max<long>(kLanesOneWavePerSimd, (long)(kLastLevelCacheBytes / table_bytes));
+  }
+  p.grid = (int)std::min<long>(p.grid, std::max<long>(1, resident / p.block));
   static const char* names[2][3] = {
       {"k_fused_per_env<4,0>", "k_fused_per_env<4,1>", "k_fused_per_env<4,2>"},
       {"k_fused_per_env<8,0>", "k_fused_per_env<8,1>", "k_fused_per_env<8,2>"}};
@@ -228,39 +249,129 @@ void launch_fused_a(const crl_engine* e, const FusedPlan& p, uint64_t t0, int n)
   }
 }
 
-int reduce_apply(crl_engine* e, float* Q, const int32_t* key, const float* delta, int n) {
-  const int grid = (int)((e->K + crl::kOwnKeys - 1) / crl::kOwnKeys);
-  hipLaunchKernelGGL(crl::k_reduce_apply, dim3(grid), dim3(crl::kReduceBlock), 0, e->stream, Q,
-                     (int)e->K, key, delta, n);
+constexpr size_t kHandoffLimitBytes = (size_t)64 << 20;
+
+int ceil_log2(size_t v) {
+  int b = 0;
+  while (((size_t)1 << b) < v) ++b;
+  return b;
+}
+
+crl::ReduceGeom reduce_geom(const crl_engine* e, int n) {
+  crl::ReduceGeom G{};
+  G.K = (int)e->K;
+  G.key_bits = std::max(1, ceil_log2(e->K));
+  G.own_shift = ceil_log2((e->K + crl::kOwnKeys - 1) / crl::kOwnKeys);
+  G.n_blocks = (n + crl::kBlockSamples - 1) / crl::kBlockSamples;
+  return G;
+}
+
+size_t handoff_records(const crl::ReduceGeom& G) {
+  return ((size_t)1 << G.own_shift) * (size_t)G.n_blocks * crl::kSlotCap;
+}
+
+// the two-pass reduction needs the dense LDS table (K <= 16384) and a bounded hand-off buffer
+bool reduce_fast(const crl_engine* e, const crl::ReduceGeom& G) {
+  return e->K <= (size_t)crl::kDenseKeys && handoff_records(G) * sizeof(uint2) <= kHandoffLimitBytes;
+}
+
+constexpr size_t kOwnersLds = (size_t)(crl::kTileBlocks + crl::kTileBlocks / crl::kGroupBlocks) *
+                              crl::kOwnKeys * sizeof(float);
+
+template <class Kern>
+hipError_t allow_lds(Kern kern, size_t bytes) {
+  return hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
+                             hipFuncAttributeMaxDynamicSharedMemorySize, (int)bytes);
+}
+
+// kernels that use more than the default 64 KB of LDS per workgroup (gfx950 has 160 KB)
+int opt_in_lds(crl_engine* e) {
+  if (e->lds_opt_in) return CRL_OK;
+  const size_t act = sizeof(crl::ReduceLds) + (size_t)kLdsMapLimitBytes;
+  HIP_TRY(allow_lds(crl::k_reduce_blocks, sizeof(crl::ReduceLds)));
+  HIP_TRY(allow_lds(crl::k_reduce_owners, kOwnersLds));
+  HIP_TRY(allow_lds(crl::k_shared_act<4, 1, true>, act));
+  HIP_TRY(allow_lds(crl::k_shared_act<4, 2, true>, act));
+  HIP_TRY(allow_lds(crl::k_shared_act<8, 1, true>, act));
+  HIP_TRY(allow_lds(crl::k_shared_act<8, 2, true>, act));
+  e->lds_opt_in = true;
+  return CRL_OK;
+}
+
+int ensure_handoff(crl_engine* e, const crl::ReduceGeom& G) {
+  const size_t recs = handoff_records(G);
+  hipError_t h = e->handoff.ensure(recs);
+  if (h == hipSuccess) h = e->handoff_count.ensure(recs / crl::kSlotCap);
+  if (h != hipSuccess) return fail(CRL_E_ALLOC, "hand-off buffer allocation failed: %s", hipGetErrorString(h));
+  return opt_in_lds(e);
+}
+
+int reduce_owners(crl_engine* e, const crl::ReduceGeom& G, float* Q, const int32_t* key,
+                  const float* delta, int n) {
+  hipLaunchKernelGGL(crl::k_reduce_owners, dim3(1 << G.own_shift), dim3(256), kOwnersLds, e->stream, G,
+                     Q, key, delta, n, e->handoff.p, e->handoff_count.p);
   HIP_TRY(hipGetLastError());
   return CRL_OK;
 }
 
-// one shared-table step: act (select+move+delta), then ordered reduce + apply
-int shared_step(crl_engine* e, uint64_t t, int trace_row) {
+// Q[k] += ordered sum of delta[i] with key[i] == k, for n samples on one table
+int reduce_apply(crl_engine* e, float* Q, const int32_t* key, const float* delta, int n) {
+  const crl::ReduceGeom G = reduce_geom(e, n);
+  if (!reduce_fast(e, G)) {
+    const int grid = (int)((e->K + crl::kOwnKeys - 1) / crl::kOwnKeys);
+    hipLaunchKernelGGL(crl::k_reduce_scan, dim3(grid), dim3(256), 0, e->stream, Q, (int)e->K, key,
+                       delta, n);
+    HIP_TRY(hipGetLastError());
+    return CRL_OK;
+  }
+  int rc = ensure_handoff(e, G);
+  if (rc) return rc;
+  hipLaunchKernelGGL(crl::k_reduce_blocks, dim3(G.n_blocks), dim3(crl::kBlockSamples),
+                     sizeof(crl::ReduceLds), e->stream, G, key, delta, n, e->handoff.p,
+                     e->handoff_count.p);
+  HIP_TRY(hipGetLastError());
+  return reduce_owners(e, G, Q, key, delta, n);
+}
+
+template <int A, int MAP>
+void launch_shared_act(crl_engine* e, bool reduce, const crl::ReduceGeom& G, uint64_t t, int trace_row) {
   const crl::Rules R = e->rules();
   const crl::Ptrs P = e->ptrs();
   const int block = 256, grid = (e->N + block - 1) / block;
+  const size_t map_lds = MAP == 1 ? (size_t)e->map_words * 4 : 0;
+  if (reduce)
+    hipLaunchKernelGGL((crl::k_shared_act<A, MAP, true>), dim3(grid), dim3(block),
+                       sizeof(crl::ReduceLds) + map_lds, e->stream, R, P, t, trace_row, e->key.p,
+                       e->delta.p, G, e->handoff.p, e->handoff_count.p);
+  else
+    hipLaunchKernelGGL((crl::k_shared_act<A, MAP, false>), dim3(grid), dim3(block), map_lds, e->stream,
+                       R, P, t, trace_row, e->key.p, e->delta.p, G, e->handoff.p, e->handoff_count.p);
+}
+
+// one shared-table step: act (select + move + delta + block sums), then the key owners
+int shared_step(crl_engine* e, uint64_t t, int trace_row) {
+  const crl::ReduceGeom G = reduce_geom(e, e->N);
+  const bool fast = reduce_fast(e, G);
+  if (fast) {
+    int rc = ensure_handoff(e, G);
+    if (rc) return rc;
+  }
   const bool lds_map =
       e->cfg.map_mode == CRL_MAP_SHARED && (size_t)e->map_words * 4 <= (size_t)kLdsMapLimitBytes;
-  const size_t lds = lds_map ? (size_t)e->map_words * 4 : 0;
   if (e->A == 4) {
-    if (lds_map)
-      hipLaunchKernelGGL((crl::k_shared_act<4, 1>), dim3(grid), dim3(block), lds, e->stream, R, P, t,
-                         trace_row, e->key.p, e->delta.p);
-    else
-      hipLaunchKernelGGL((crl::k_shared_act<4, 2>), dim3(grid), dim3(block), 0, e->stream, R, P, t,
-                         trace_row, e->key.p, e->delta.p);
+    if (lds_map) launch_shared_act<4, 1>(e, fast, G, t, trace_row);
+    else launch_shared_act<4, 2>(e, fast, G, t, trace_row);
   } else {
-    if (lds_map)
-      hipLaunchKernelGGL((crl::k_shared_act<8, 1>), dim3(grid), dim3(block), lds, e->stream, R, P, t,
-                         trace_row, e->key.p, e->delta.p);
-    else
-      hipLaunchKernelGGL((crl::k_shared_act<8, 2>), dim3(grid), dim3(block), 0, e->stream, R, P, t,
-                         trace_row, e->key.p, e->delta.p);
+    if (lds_map) launch_shared_act<8, 1>(e, fast, G, t, trace_row);
+    else launch_shared_act<8, 2>(e, fast, G, t, trace_row);
   }
   HIP_TRY(hipGetLastError());
-  return reduce_apply(e, e->Q.p, e->key.p, e->delta.p, e->N);
+  if (fast) return reduce_owners(e, G, e->Q.p, e->key.p, e->delta.p, e->N);
+  const int grid = (int)((e->K + crl::kOwnKeys - 1) / crl::kOwnKeys);
+  hipLaunchKernelGGL(crl::k_reduce_scan, dim3(grid), dim3(256), 0, e->stream, e->Q.p, (int)e->K,
+                     e->key.p, e->delta.p, e->N);
+  HIP_TRY(hipGetLastError());
+  return CRL_OK;
 }
 
 int check_engine(const crl_engine* e) {
@@ -408,6 +519,13 @@ int crl_set_stream(crl_engine* e, void* hip_stream) {
   if (rc) return rc;
   HIP_TRY(hipStreamSynchronize(e->stream));
   e->stream = reinterpret_cast<hipStream_t>(hip_stream);
+  return CRL_OK;
+}
+
+int crl_set_resident_envs(crl_engine* e, int32_t n_envs) {
+  if (!e) return fail(CRL_E_ARG, "null engine");
+  if (n_envs < 0) return fail(CRL_E_ARG, "negative env count");
+  e->resident_envs = n_envs;
   return CRL_OK;
 }
 
@@ -781,7 +899,7 @@ int crl_fused_kernel_info(crl_engine* e, char* name, size_t name_len, int32_t* g
     if (block) *block = p.block;
     if (lds_bytes) *lds_bytes = (int32_t)p.lds;
   } else {
-    if (name && name_len) snprintf(name, name_len, "k_shared_act+k_reduce_apply");
+    if (name && name_len) snprintf(name, name_len, "k_shared_act+k_reduce_owners");
     if (grid) *grid = (e->N + 255) / 256;
     if (block) *block = 256;
     if (lds_bytes) *lds_bytes = e->map_words * 4;

@@ -94,7 +94,8 @@ struct WordStream {
       blk = philox4x32_10(a, id, b, 0u, (uint32_t)seed, (uint32_t)(seed >> 32));
       cached_block = b;
     }
-    return blk.w[i & 3];
+    const uint32_t w[4] = {blk.w0, blk.w1, blk.w2, blk.w3};
+    return w[i & 3];
   }
 };
 
@@ -130,14 +131,17 @@ extern "C" {
 
 void crl_philox4x32_10(const uint32_t ctr[4], const uint32_t key[2], uint32_t out[4]) {
   const crl::Philox4 r = crl::philox4x32_10(ctr[0], ctr[1], ctr[2], ctr[3], key[0], key[1]);
-  for (int i = 0; i < 4; ++i) out[i] = r.w[i];
+  out[0] = r.w0;
+  out[1] = r.w1;
+  out[2] = r.w2;
+  out[3] = r.w3;
 }
 
 void crl_explore_draw(uint64_t seed, uint32_t env, uint64_t t, int32_t n_actions, float* u,
                       int32_t* a_rand) {
   const crl::Philox4 b = crl::explore_block(seed, env, t >> 1);
-  const uint32_t w0 = (t & 1) ? b.w[2] : b.w[0];
-  const uint32_t w1 = (t & 1) ? b.w[3] : b.w[1];
+  const uint32_t w0 = (t & 1) ? b.w2 : b.w0;
+  const uint32_t w1 = (t & 1) ? b.w3 : b.w1;
   if (u) *u = crl::u01(w0);
   if (a_rand) *a_rand = (int32_t)crl::below(w1, (uint32_t)n_actions);
 }

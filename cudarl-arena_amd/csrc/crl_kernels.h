@@ -11,6 +11,7 @@
 // HBM traffic or by dependent-access latency.
 #pragma once
 #include "crl_device.h"
+#include "crl_reduce.h"
 
 namespace crl {
 
@@ -51,9 +52,9 @@ struct Draw {
   int a;
 };
 
-__device__ __forceinline__ Draw pick_draw(const Philox4& blk, uint64_t t, int A) {
-  const uint32_t w0 = (t & 1) ? blk.w[2] : blk.w[0];
-  const uint32_t w1 = (t & 1) ? blk.w[3] : blk.w[1];
+__device__ __forceinline__ Draw pick_draw(const Philox4 blk, uint64_t t, int A) {
+  const uint32_t w0 = (t & 1) ? blk.w2 : blk.w0;
+  const uint32_t w1 = (t & 1) ? blk.w3 : blk.w1;
   Draw d;
   d.u = u01(w0);
   d.a = (int)below(w1, (uint32_t)A);
@@ -77,107 +78,121 @@ __global__ __launch_bounds__(256) void k_fused_per_env(const Rules R, const Ptrs
   extern __shared__ uint32_t lds[];
   const int tid = threadIdx.x;
   const int bdim = blockDim.x;
-  const int env0 = blockIdx.x * bdim;
-  const int env = env0 + tid;
-  const bool live = env < P.N;
+  const int n_chunks = (P.N + bdim - 1) / bdim;
 
-  if (MAP == 0) {
-    // the block's maps are contiguous in HBM: coalesced read, transposing write
-    const int n_here = min(bdim, P.N - env0);
-    const uint32_t* src = P.map + (size_t)env0 * P.map_words;
-    const int total = n_here * P.map_words;
-    for (int i = tid; i < total; i += bdim) {
-      const int e = i / P.map_words, w = i - e * P.map_words;
-      lds[w * bdim + e] = src[i];
-    }
-    __syncthreads();
-  } else if (MAP == 1) {
+  if (MAP == 1) {
     for (int i = tid; i < P.map_words; i += bdim) lds[i] = P.map[i];
     __syncthreads();
   }
-  if (!live) return;
 
-  const uint32_t* gmap = P.map + (P.map_shared ? 0 : (size_t)env * P.map_words);
-  auto cls = [&](int cell) -> int {
-    uint32_t word;
-    if (MAP == 0)
-      word = lds[(cell >> 4) * bdim + tid];
-    else if (MAP == 1)
-      word = lds[cell >> 4];
-    else
-      word = gmap[cell >> 4];
-    return cell_class_of(word, cell);
-  };
-  const float* cr = P.cell_reward ? P.cell_reward + (P.map_shared ? 0 : (size_t)env * P.S) : nullptr;
+  // A block takes chunks blockIdx, blockIdx + gridDim, ... and runs each for all
+  // n_steps.  The grid size therefore sets how many envs (and how many bytes of
+  // their tables) are live on the chip at once: small enough and the rows an
+  // env keeps returning to are still in the last-level cache.
+  for (int chunk = blockIdx.x; chunk < n_chunks; chunk += gridDim.x) {
+    const int env0 = chunk * bdim;
+    const int env = env0 + tid;
+    const bool live = env < P.N;
 
-  float* __restrict__ Qe = P.Q + (size_t)env * P.S * A;
-  const int start = P.start[env];
-  const int sx = start % R.W, sy = start / R.W;
-  int s = P.s[env];
-  int x = s % R.W, y = s / R.W;
-  int ep_step = P.ep_step[env];
-  int episode = P.episode[env];
-  bool done = P.done[env] != 0;
-  float reward = 0.0f;
-  int action = 0;
-  Row<A> row = load_row<A>(Qe + (size_t)s * A);
-  Philox4 blk = explore_block(R.seed, (uint32_t)env, t0 >> 1);
-
-  for (int k = 0; k < n_steps; ++k) {
-    const uint64_t t = t0 + (uint64_t)k;
-    if (k > 0 && (t & 1) == 0) blk = explore_block(R.seed, (uint32_t)env, t >> 1);
-    Draw d = pick_draw(blk, t, A);
-    if (P.u_sup && t >= P.sup_t0 && t - P.sup_t0 < (uint64_t)P.sup_n) {
-      const size_t o = (size_t)(t - P.sup_t0) * P.N + env;
-      d.u = P.u_sup[o];
-      d.a = P.a_sup[o];
+    if (MAP == 0) {
+      __syncthreads();  // the previous chunk's readers are done with the map
+      // the chunk's maps are contiguous in HBM: coalesced read, transposing write
+      const int n_here = min(bdim, P.N - env0);
+      const uint32_t* src = P.map + (size_t)env0 * P.map_words;
+      const int total = n_here * P.map_words;
+      for (int i = tid; i < total; i += bdim) {
+        const int e = i / P.map_words, w = i - e * P.map_words;
+        lds[w * bdim + e] = src[i];
+      }
+      __syncthreads();
     }
-    const float eps = eps_of(R, P.eps_tab, t, episode);
-    const int a = (d.u < eps) ? d.a : row_argmax<A>(row);
+    if (!live) continue;  // only in the last chunk, after its barriers
 
-    const int s0 = s;
-    bool hit;
-    step_rule(R, cls, cr, x, y, a, reward, hit);
-    const int s2 = y * R.W + x;
-    done = hit || (!R.auto_reset && done);
+    const uint32_t* gmap = P.map + (P.map_shared ? 0 : (size_t)env * P.map_words);
+    auto cls = [&](int cell) -> int {
+      uint32_t word;
+      if (MAP == 0)
+        word = lds[(cell >> 4) * bdim + tid];
+      else if (MAP == 1)
+        word = lds[cell >> 4];
+      else
+        word = gmap[cell >> 4];
+      return cell_class_of(word, cell);
+    };
+    const float* cr =
+        P.cell_reward ? P.cell_reward + (P.map_shared ? 0 : (size_t)env * P.S) : nullptr;
 
-    // Q row of the new cell; when the env did not move it is the row in registers
-    Row<A> row2 = row;
-    if (s2 != s0) row2 = load_row<A>(Qe + (size_t)s2 * A);
-    const float m = row_max<A>(row2, done, R.max_mode);
-    const float qn = td_value(row_get<A>(row, a), reward, m, R.lr, R.gamma);
-    Qe[(size_t)s0 * A + a] = qn;
-    if (s2 == s0) row_set<A>(row2, a, qn);
+    float* __restrict__ Qe = P.Q + (size_t)env * P.S * A;
+    const int start = P.start[env];
+    const int sx = start % R.W, sy = start / R.W;
+    int s = P.s[env];
+    int x = s % R.W, y = s / R.W;
+    int ep_step = P.ep_step[env];
+    int episode = P.episode[env];
+    bool done = P.done[env] != 0;
+    float reward = 0.0f;
+    int action = 0;
+    Row<A> row = load_row<A>(Qe + (size_t)s * A);
+    Philox4 blk = explore_block(R.seed, (uint32_t)env, t0 >> 1);
 
-    ep_step += 1;
-    action = a;
-    if (env < P.trace_n && P.trace_cursor + k < P.trace_cap) {
-      const size_t o = (size_t)(P.trace_cursor + k) * P.trace_n + env;
-      P.tr_s[o] = s2;
-      P.tr_a[o] = (uint8_t)a;
-      P.tr_r[o] = reward;
-      P.tr_d[o] = done ? 1 : 0;
+    for (int k = 0; k < n_steps; ++k) {
+      const uint64_t t = t0 + (uint64_t)k;
+      Draw d = pick_draw(blk, t, A);
+      if (P.u_sup && t >= P.sup_t0 && t - P.sup_t0 < (uint64_t)P.sup_n) {
+        const size_t o = (size_t)(t - P.sup_t0) * P.N + env;
+        d.u = P.u_sup[o];
+        d.a = P.a_sup[o];
+      }
+      const float eps = eps_of(R, P.eps_tab, t, episode);
+      const int a = (d.u < eps) ? d.a : row_argmax(row);
+
+      const int s0 = s;
+      bool hit;
+      step_rule(R, cls, cr, x, y, a, reward, hit);
+      const int s2 = y * R.W + x;
+      done = hit || (!R.auto_reset && done);
+
+      // Q row of the new cell; when the env did not move it is the row in registers
+      Row<A> row2 = row;
+      if (s2 != s0) row2 = load_row<A>(Qe + (size_t)s2 * A);
+      // the next step's draws depend on nothing: the Philox rounds run while the
+      // row load is in flight
+      if ((t & 1) == 1) blk = explore_block(R.seed, (uint32_t)env, (t + 1) >> 1);
+      const float m = row_max(row2, done, R.max_mode);
+      const float qn = td_value(row_get(row, a), reward, m, R.lr, R.gamma);
+      Qe[(size_t)s0 * A + a] = qn;
+      if (s2 == s0) row2 = row_set(row2, a, qn);
+
+      ep_step += 1;
+      action = a;
+      if (env < P.trace_n && P.trace_cursor + k < P.trace_cap) {
+        const size_t o = (size_t)(P.trace_cursor + k) * P.trace_n + env;
+        P.tr_s[o] = s2;
+        P.tr_a[o] = (uint8_t)a;
+        P.tr_r[o] = reward;
+        P.tr_d[o] = done ? 1 : 0;
+      }
+      if (R.auto_reset && (done || (R.episode_len > 0 && ep_step >= R.episode_len))) {
+        x = sx;
+        y = sy;
+        s = start;
+        ep_step = 0;
+        episode += 1;
+        row = load_row<A>(Qe + (size_t)start * A);
+        if (start == s0) row = row_set(row, a, qn);  // the value just written, from registers
+      } else {
+        s = s2;
+        row = row2;
+      }
     }
-    if (R.auto_reset && (done || (R.episode_len > 0 && ep_step >= R.episode_len))) {
-      x = sx;
-      y = sy;
-      s = start;
-      ep_step = 0;
-      episode += 1;
-      row = load_row<A>(Qe + (size_t)start * A);
-      if (start == s0) row_set<A>(row, a, qn);  // the value just written, from registers
-    } else {
-      s = s2;
-      row = row2;
-    }
+
+    P.s[env] = s;
+    P.ep_step[env] = ep_step;
+    P.episode[env] = episode;
+    P.reward[env] = reward;
+    P.done[env] = done ? 1 : 0;
+    P.action[env] = (uint8_t)action;
   }
-
-  P.s[env] = s;
-  P.ep_step[env] = ep_step;
-  P.episode[env] = episode;
-  P.reward[env] = reward;
-  P.done[env] = done ? 1 : 0;
-  P.action[env] = (uint8_t)action;
 }
 
 // ---------------------------------------------------------------------------
@@ -295,7 +310,7 @@ __global__ __launch_bounds__(256) void k_update_per_env(const Rules R, const Ptr
   const int s = T.s[env], a = T.a[env], s2 = T.s2[env];
   if ((unsigned)a >= (unsigned)A) return;  // an invalid action has no table entry
   const Row<A> row2 = load_row<A>(Qe + (size_t)s2 * A);
-  const float m = row_max<A>(row2, T.done[env] != 0, R.max_mode);
+  const float m = row_max(row2, T.done[env] != 0, R.max_mode);
   const size_t k = (size_t)s * A + a;
   Qe[k] = td_value(Qe[k], T.r[env], m, R.lr, R.gamma);
 }
@@ -321,138 +336,93 @@ __global__ __launch_bounds__(256) void k_delta(const float* __restrict__ Q, cons
     return;
   }
   const Row<A> row2 = load_row<A>(Q + (size_t)s2[i] * A);
-  const float m = row_max<A>(row2, done[i] != 0, max_mode);
+  const float m = row_max(row2, done[i] != 0, max_mode);
   const int k = s[i] * A + ai;
   key[i] = k;
   delta[i] = td_delta(Q[k], r[i], m, lr, gamma);
 }
 
 // Shared table, first half of a fused step: every env selects, moves and emits
-// (key, delta) against the table as it stands; nothing is written to Q.
+// (key, delta) against the table as it stands; nothing is written to Q.  With
+// REDUCE the workgroup (= one 256-sample block of the ordered reduction) also
+// folds its own deltas and hands the block sums to the key owners.
 // MAP = 1: shared map staged in LDS; MAP = 2: maps in global memory.
-template <int A, int MAP>
+template <int A, int MAP, bool REDUCE>
 __global__ __launch_bounds__(256) void k_shared_act(const Rules R, const Ptrs P, const uint64_t t,
                                                      const int trace_row,
                                                      int32_t* __restrict__ key,
-                                                     float* __restrict__ delta) {
-  extern __shared__ uint32_t lds[];
+                                                     float* __restrict__ delta, const ReduceGeom G,
+                                                     uint2* __restrict__ handoff,
+                                                     uint8_t* __restrict__ handoff_count) {
+  extern __shared__ unsigned char lds_raw[];
+  uint32_t* lds_map = reinterpret_cast<uint32_t*>(lds_raw + (REDUCE ? sizeof(ReduceLds) : 0));
   const int tid = threadIdx.x;
   const int env = blockIdx.x * blockDim.x + tid;
   if (MAP == 1) {
-    for (int i = tid; i < P.map_words; i += blockDim.x) lds[i] = P.map[i];
+    for (int i = tid; i < P.map_words; i += blockDim.x) lds_map[i] = P.map[i];
     __syncthreads();
   }
-  if (env >= P.N) return;
-  const uint32_t* gmap = P.map + (P.map_shared ? 0 : (size_t)env * P.map_words);
-  auto cls = [&](int cell) -> int {
-    const uint32_t word = (MAP == 1) ? lds[cell >> 4] : gmap[cell >> 4];
-    return cell_class_of(word, cell);
-  };
-  const float* cr = P.cell_reward ? P.cell_reward + (P.map_shared ? 0 : (size_t)env * P.S) : nullptr;
-  const float* __restrict__ Q = P.Q;
+  const bool live = env < P.N;
+  int my_key = 0;
+  float my_delta = 0.0f;
+  if (live) {
+    const uint32_t* gmap = P.map + (P.map_shared ? 0 : (size_t)env * P.map_words);
+    auto cls = [&](int cell) -> int {
+      const uint32_t word = (MAP == 1) ? lds_map[cell >> 4] : gmap[cell >> 4];
+      return cell_class_of(word, cell);
+    };
+    const float* cr =
+        P.cell_reward ? P.cell_reward + (P.map_shared ? 0 : (size_t)env * P.S) : nullptr;
+    const float* __restrict__ Q = P.Q;
 
-  const int s0 = P.s[env];
-  int x = s0 % R.W, y = s0 / R.W;
-  const Row<A> row = load_row<A>(Q + (size_t)s0 * A);
-  Draw d = pick_draw(explore_block(R.seed, (uint32_t)env, t >> 1), t, A);
-  if (P.u_sup && t >= P.sup_t0 && t - P.sup_t0 < (uint64_t)P.sup_n) {
-    const size_t o = (size_t)(t - P.sup_t0) * P.N + env;
-    d.u = P.u_sup[o];
-    d.a = P.a_sup[o];
-  }
-  const int episode = P.episode[env];
-  const float eps = eps_of(R, P.eps_tab, t, episode);
-  const int a = (d.u < eps) ? d.a : row_argmax<A>(row);
-  float reward;
-  bool hit;
-  step_rule(R, cls, cr, x, y, a, reward, hit);
-  const int s2 = y * R.W + x;
-  const bool done = hit || (!R.auto_reset && P.done[env] != 0);
-  const Row<A> row2 = load_row<A>(Q + (size_t)s2 * A);
-  const float m = row_max<A>(row2, done, R.max_mode);
-  key[env] = s0 * A + a;
-  delta[env] = td_delta(row_get<A>(row, a), reward, m, R.lr, R.gamma);
-
-  const int ep_step = P.ep_step[env] + 1;
-  P.reward[env] = reward;
-  P.done[env] = done ? 1 : 0;
-  P.action[env] = (uint8_t)a;
-  if (env < P.trace_n && trace_row < P.trace_cap) {
-    const size_t o = (size_t)trace_row * P.trace_n + env;
-    P.tr_s[o] = s2;
-    P.tr_a[o] = (uint8_t)a;
-    P.tr_r[o] = reward;
-    P.tr_d[o] = done ? 1 : 0;
-  }
-  if (R.auto_reset && (done || (R.episode_len > 0 && ep_step >= R.episode_len))) {
-    P.s[env] = P.start[env];
-    P.ep_step[env] = 0;
-    P.episode[env] = episode + 1;
-  } else {
-    P.s[env] = s2;
-    P.ep_step[env] = ep_step;
-  }
-}
-
-// ---------------------------------------------------------------------------
-// Deterministic segmented reduction: Q[k] = Q[k] + sum of delta[i] over the i
-// with key[i] == k, added strictly in increasing i from +0.0f - no float
-// atomics.  Each workgroup owns kOwnKeys consecutive keys and scans the whole
-// key array: its four waves take consecutive quarters of a segment, each
-// compacts its matches in lane order into an LDS list (ballot + prefix count),
-// and wave 0 then folds the four lists in order, one lane per owned key.
-// ---------------------------------------------------------------------------
-constexpr int kOwnKeys = 64;
-constexpr int kReduceBlock = 256;
-constexpr int kWaveSpan = 1024;                // entries one wave scans per segment
-constexpr int kSegment = 4 * kWaveSpan;        // entries per segment
-
-__global__ __launch_bounds__(kReduceBlock) void k_reduce_apply(float* __restrict__ Q, const int K,
-                                                                const int32_t* __restrict__ key,
-                                                                const float* __restrict__ delta,
-                                                                const int n) {
-  __shared__ float l_d[4][kWaveSpan];
-  __shared__ uint8_t l_k[4][kWaveSpan];
-  __shared__ int l_cnt[4];
-  const int tid = threadIdx.x;
-  const int lane = tid & 63;
-  const int wave = tid >> 6;
-  const int owner = blockIdx.x;
-  float acc = 0.0f;
-
-  for (int seg = 0; seg < n; seg += kSegment) {
-    int cnt = 0;
-    const int base = seg + wave * kWaveSpan;
-#pragma unroll 4
-    for (int it = 0; it < kWaveSpan / 64; ++it) {
-      const int i = base + it * 64 + lane;
-      const int k = (i < n) ? key[i] : -1;
-      const bool match = (k >= 0) && ((k / kOwnKeys) == owner);
-      const unsigned long long bal = __ballot(match);
-      if (bal != 0ull) {
-        if (match) {
-          const int pos = cnt + __popcll(bal & ((1ull << lane) - 1ull));
-          l_d[wave][pos] = delta[i];
-          l_k[wave][pos] = (uint8_t)(k - owner * kOwnKeys);
-        }
-        cnt += __popcll(bal);
-      }
+    const int s0 = P.s[env];
+    int x = s0 % R.W, y = s0 / R.W;
+    const Row<A> row = load_row<A>(Q + (size_t)s0 * A);
+    Draw d = pick_draw(explore_block(R.seed, (uint32_t)env, t >> 1), t, A);
+    if (P.u_sup && t >= P.sup_t0 && t - P.sup_t0 < (uint64_t)P.sup_n) {
+      const size_t o = (size_t)(t - P.sup_t0) * P.N + env;
+      d.u = P.u_sup[o];
+      d.a = P.a_sup[o];
     }
-    if (lane == 0) l_cnt[wave] = cnt;
-    __syncthreads();
-    if (wave == 0) {
-      for (int w = 0; w < 4; ++w) {
-        const int c = l_cnt[w];
-        for (int e = 0; e < c; ++e) {
-          const float dv = l_d[w][e];
-          if (l_k[w][e] == lane) acc = acc + dv;
-        }
-      }
+    const int episode = P.episode[env];
+    const float eps = eps_of(R, P.eps_tab, t, episode);
+    const int a = (d.u < eps) ? d.a : row_argmax(row);
+    float reward;
+    bool hit;
+    step_rule(R, cls, cr, x, y, a, reward, hit);
+    const int s2 = y * R.W + x;
+    const bool done = hit || (!R.auto_reset && P.done[env] != 0);
+    const Row<A> row2 = load_row<A>(Q + (size_t)s2 * A);
+    const float m = row_max(row2, done, R.max_mode);
+    my_key = s0 * A + a;
+    my_delta = td_delta(row_get(row, a), reward, m, R.lr, R.gamma);
+    key[env] = my_key;
+    delta[env] = my_delta;
+
+    const int ep_step = P.ep_step[env] + 1;
+    P.reward[env] = reward;
+    P.done[env] = done ? 1 : 0;
+    P.action[env] = (uint8_t)a;
+    if (env < P.trace_n && trace_row < P.trace_cap) {
+      const size_t o = (size_t)trace_row * P.trace_n + env;
+      P.tr_s[o] = s2;
+      P.tr_a[o] = (uint8_t)a;
+      P.tr_r[o] = reward;
+      P.tr_d[o] = done ? 1 : 0;
     }
-    __syncthreads();
+    if (R.auto_reset && (done || (R.episode_len > 0 && ep_step >= R.episode_len))) {
+      P.s[env] = P.start[env];
+      P.ep_step[env] = 0;
+      P.episode[env] = episode + 1;
+    } else {
+      P.s[env] = s2;
+      P.ep_step[env] = ep_step;
+    }
   }
-  const int k = owner * kOwnKeys + lane;
-  if (wave == 0 && k < K) Q[k] = Q[k] + acc;
+  if (REDUCE) {
+    ReduceLds& L = *reinterpret_cast<ReduceLds*>(lds_raw);
+    reduce_block(L, G, blockIdx.x, my_key, my_delta, live, handoff, handoff_count);
+  }
 }
 
 // plain copy of n16 16-byte words: the known-size launch that calibrates the

@@ -14,8 +14,10 @@
 
 namespace crl {
 
+// four named words, not an array: a select between two array elements would be
+// folded into an indexed load and push the block into scratch memory on the GPU
 struct Philox4 {
-  uint32_t w[4];
+  uint32_t w0, w1, w2, w3;
 };
 
 CRL_HD Philox4 philox4x32_10(uint32_t c0, uint32_t c1, uint32_t c2, uint32_t c3, uint32_t k0,
@@ -34,10 +36,10 @@ CRL_HD Philox4 philox4x32_10(uint32_t c0, uint32_t c1, uint32_t c2, uint32_t c3,
     k1 += 0xBB67AE85u;
   }
   Philox4 r;
-  r.w[0] = c0;
-  r.w[1] = c1;
-  r.w[2] = c2;
-  r.w[3] = c3;
+  r.w0 = c0;
+  r.w1 = c1;
+  r.w2 = c2;
+  r.w3 = c3;
   return r;
 }
 

@@ -115,6 +115,11 @@ int crl_destroy(crl_engine* e);
 /* Use `hip_stream` (a hipStream_t, NULL = the null stream) for all later work. */
 int crl_set_stream(crl_engine* e, void* hip_stream);
 int crl_sync(crl_engine* e);
+/* Tuning (no reference counterpart): how many envs crl_run_fused keeps in
+ * flight at once for per-env tables; the rest follow in turn inside the same
+ * launch.  0 = automatic (as many as keep the tables in the last-level cache).
+ * Results do not depend on it. */
+int crl_set_resident_envs(crl_engine* e, int32_t n_envs);
 
 /* -- maps ------------------------------------------------------------------ */
 

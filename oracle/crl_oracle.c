@@ -25,7 +25,8 @@
  *   orc_run + eps schedule        training.log:24931-24953 (returns -5.00 / -10.00,
  *                                 epsilon 0.082, 0.007, 0.001)
  *   ordered reduction (shared)    defined here, not by the reference: brute force
- *                                 against a dictionary-of-lists summation
+ *                                 of the definition key by key, and (up to 256
+ *                                 samples) a dictionary-of-lists summation
  */
 #include <math.h>
 #include <stdint.h>
@@ -266,25 +267,149 @@ void orc_td_update_one(float* Q, int A, int s, int a, float r, int s2, int done,
   Q[(size_t)s * A + a] = orc_td_value(Q[(size_t)s * A + a], r, m, lr, gamma);
 }
 
-/* Batch on one table of K = S*A entries: every read sees the table before the
- * call; deltas of equal (s,a) are added in sample order, left to right,
- * starting from +0.0f; then Q[k] = Q[k] + sum[k] for every k.  (The
- * reference's kernel races on duplicates, src/kernels.cu:114; this is the
- * build's deterministic rule and equals the reference up to one rounding when
- * every (s,a) is unique and no written row is another sample's next row.) */
+/* ---- R1: the ordered sum of deltas that hit the same (s,a) ----------------- */
+/*
+ * Nothing like it exists in the reference (its kernel races on duplicates,
+ * src/kernels.cu:114); the order is this build's definition.  Samples (envs)
+ * are taken in index order through a fixed three-level tree:
+ *
+ *   block  = 256 consecutive samples, added left to right from +0.0f
+ *   group  = 16 consecutive blocks, block sums added left to right from +0.0f
+ *   total  = group sums added left to right from +0.0f
+ *   Q[k]   = Q[k] + total[k]   for every k
+ *
+ * A block or group that holds no sample of a key contributes +0.0f, which
+ * changes nothing (a running sum that starts at +0.0f is never -0.0f), so the
+ * implementation below only visits the keys a block / group touched.  With at
+ * most 256 samples this is plain left-to-right summation.
+ */
+enum { ORC_BLOCK = 256, ORC_GROUP = 16 };
+
+typedef struct {
+  size_t K;
+  float *bsum, *gsum, *total;
+  int32_t *btouch, *gtouch; /* keys touched in the open block / group */
+  uint8_t *bflag, *gflag;
+  int nb_touch, ng_touch;
+  int in_block, blocks_in_group;
+} orc_tree;
+
+static int tree_init(orc_tree* t, size_t K) {
+  memset(t, 0, sizeof *t);
+  t->K = K;
+  t->bsum = (float*)calloc(K, sizeof(float));
+  t->gsum = (float*)calloc(K, sizeof(float));
+  t->total = (float*)calloc(K, sizeof(float));
+  t->btouch = (int32_t*)malloc(ORC_BLOCK * sizeof(int32_t));
+  t->gtouch = (int32_t*)malloc((size_t)ORC_BLOCK * ORC_GROUP * sizeof(int32_t));
+  t->bflag = (uint8_t*)calloc(K, 1);
+  t->gflag = (uint8_t*)calloc(K, 1);
+  return (t->bsum && t->gsum && t->total && t->btouch && t->gtouch && t->bflag && t->gflag) ? 0 : -3;
+}
+
+static void tree_free(orc_tree* t) {
+  free(t->bsum); free(t->gsum); free(t->total);
+  free(t->btouch); free(t->gtouch); free(t->bflag); free(t->gflag);
+}
+
+static void tree_close_group(orc_tree* t) {
+  for (int i = 0; i < t->ng_touch; ++i) {
+    int32_t k = t->gtouch[i];
+    t->total[k] = t->total[k] + t->gsum[k];
+    t->gsum[k] = 0.0f;
+    t->gflag[k] = 0;
+  }
+  t->ng_touch = 0;
+  t->blocks_in_group = 0;
+}
+
+static void tree_close_block(orc_tree* t) {
+  for (int i = 0; i < t->nb_touch; ++i) {
+    int32_t k = t->btouch[i];
+    t->gsum[k] = t->gsum[k] + t->bsum[k];
+    t->bsum[k] = 0.0f;
+    t->bflag[k] = 0;
+    if (!t->gflag[k]) {
+      t->gflag[k] = 1;
+      t->gtouch[t->ng_touch++] = k;
+    }
+  }
+  t->nb_touch = 0;
+  t->in_block = 0;
+  if (++t->blocks_in_group == ORC_GROUP) tree_close_group(t);
+}
+
+/* next sample in index order; key < 0 means the sample carries no delta */
+static void tree_add(orc_tree* t, int64_t key, float d) {
+  if (key >= 0) {
+    t->bsum[key] = t->bsum[key] + d;
+    if (!t->bflag[key]) {
+      t->bflag[key] = 1;
+      t->btouch[t->nb_touch++] = (int32_t)key;
+    }
+  }
+  if (++t->in_block == ORC_BLOCK) tree_close_block(t);
+}
+
+/* close what is open, apply to Q, and leave the tree empty for the next pass */
+static void tree_apply(orc_tree* t, float* Q) {
+  if (t->in_block) tree_close_block(t);
+  if (t->blocks_in_group) tree_close_group(t);
+  for (size_t k = 0; k < t->K; ++k) {
+    Q[k] = Q[k] + t->total[k];
+    t->total[k] = 0.0f;
+  }
+}
+
+/* The same sums by the definition, key by key (quadratic: tests only). */
+int orc_tree_sum_bruteforce(const int32_t* key, const float* d, int n, int K, float* total) {
+  for (int k = 0; k < K; ++k) {
+    float tot = 0.0f;
+    for (int g0 = 0; g0 < n; g0 += ORC_BLOCK * ORC_GROUP) {
+      float gs = 0.0f;
+      for (int b0 = g0; b0 < n && b0 < g0 + ORC_BLOCK * ORC_GROUP; b0 += ORC_BLOCK) {
+        float bs = 0.0f;
+        for (int i = b0; i < n && i < b0 + ORC_BLOCK; ++i)
+          if (key[i] == k) bs = bs + d[i];
+        gs = gs + bs;
+      }
+      tot = tot + gs;
+    }
+    total[k] = tot;
+  }
+  return 0;
+}
+
+/* The tree of the implementation above, exposed for the same test. */
+int orc_tree_sum(const int32_t* key, const float* d, int n, int K, float* total) {
+  orc_tree t;
+  if (tree_init(&t, (size_t)K)) { tree_free(&t); return -3; }
+  for (int i = 0; i < n; ++i) tree_add(&t, key[i], d[i]);
+  for (int k = 0; k < K; ++k) total[k] = 0.0f;
+  tree_apply(&t, total); /* 0 + total */
+  tree_free(&t);
+  return 0;
+}
+
+/* Batch on one table of K = S*A entries (CudaQLearning::update_batch,
+ * src/q_learning.cu:108-174): every read sees the table before the call; the
+ * deltas are summed per (s,a) through the tree above in sample order and then
+ * applied.  Equals the reference up to one rounding when every (s,a) is unique
+ * and no written row is another sample's next row.  An action outside [0,A)
+ * has no table entry and is skipped. */
 int orc_td_update_batch(float* Q, int S, int A, int n, const int32_t* s, const int32_t* a,
                         const float* r, const int32_t* s2, const uint8_t* done, float lr,
                         float gamma, int mode) {
-  size_t K = (size_t)S * A;
-  float* sum = (float*)calloc(K, sizeof(float));
-  if (!sum) return -3;
+  orc_tree t;
+  if (tree_init(&t, (size_t)S * A)) { tree_free(&t); return -3; }
   for (int i = 0; i < n; ++i) {
+    if (a[i] < 0 || a[i] >= A) { tree_add(&t, -1, 0.0f); continue; }
     float m = orc_next_max(Q + (size_t)s2[i] * A, A, done[i], mode);
     size_t k = (size_t)s[i] * A + a[i];
-    sum[k] = sum[k] + orc_td_delta(Q[k], r[i], m, lr, gamma);
+    tree_add(&t, (int64_t)k, orc_td_delta(Q[k], r[i], m, lr, gamma));
   }
-  for (size_t k = 0; k < K; ++k) Q[k] = Q[k] + sum[k];
-  free(sum);
+  tree_apply(&t, Q);
+  tree_free(&t);
   return 0;
 }
 
@@ -332,10 +457,10 @@ static int eps_cap(const orc_config* c) {
 }
 
 /* One env, one step: select (src/train.py:200) -> step (:201) -> update (:205).
- * q is the env's table (or the shared one); with sum != NULL the delta is
- * accumulated there instead of being applied.  Returns s' before any restart. */
+ * q is the env's table (or the shared one); with sum != NULL the delta goes
+ * into the ordered tree instead of being applied.  Returns s' before any restart. */
 static int32_t env_step(const orc_config* c, float eps, float u, int32_t ar, const uint8_t* m_cls,
-                        const float* m_cr, float* q, float* sum, int32_t start, int32_t* s,
+                        const float* m_cr, float* q, orc_tree* sum, int32_t start, int32_t* s,
                         int32_t* ep_step, int32_t* episode, float* reward, uint8_t* done,
                         uint8_t* action) {
   const int A = c->n_actions;
@@ -348,7 +473,7 @@ static int32_t env_step(const orc_config* c, float eps, float u, int32_t ar, con
   float mx = orc_next_max(q + (size_t)s2 * A, A, d, c->max_mode);
   size_t key = (size_t)s0 * A + a;
   if (sum)
-    sum[key] = sum[key] + orc_td_delta(q[key], r, mx, c->lr, c->gamma);
+    tree_add(sum, (int64_t)key, orc_td_delta(q[key], r, mx, c->lr, c->gamma));
   else
     q[key] = orc_td_value(q[key], r, mx, c->lr, c->gamma);
   *ep_step += 1;
@@ -373,8 +498,8 @@ static int32_t env_step(const orc_config* c, float eps, float u, int32_t ar, con
  * Trace arrays (optional) are [n_steps][trace_n].
  *
  * Shared table: every env of a step reads the table as it was before the
- * step; the deltas are then summed per (s,a) in env order, left to right from
- * +0.0f, and Q[k] = Q[k] + sum[k] for every k.
+ * step; the deltas are then summed per (s,a) in env order through the
+ * block / group tree defined above, and Q[k] = Q[k] + total[k] for every k.
  */
 int orc_run(const orc_config* c, const uint8_t* cls, const float* cr, const int32_t* start,
             float* Q, int32_t* s, int32_t* ep_step, int32_t* episode, float* reward,
@@ -387,18 +512,18 @@ int orc_run(const orc_config* c, const uint8_t* cls, const float* cr, const int3
   const int shared = c->table_mode == 1;
   int cap = eps_cap(c);
   float* tab = (float*)malloc((size_t)cap * sizeof(float));
-  float* sum = shared ? (float*)malloc(K * sizeof(float)) : NULL;
-  if (!tab || (shared && !sum)) {
+  orc_tree tree;
+  memset(&tree, 0, sizeof tree);
+  if (!tab || (shared && tree_init(&tree, K))) {
     free(tab);
-    free(sum);
+    tree_free(&tree);
     return -3;
   }
+  orc_tree* sum = shared ? &tree : NULL;
   int len = orc_eps_table(c, tab, cap);
 
   for (int k = 0; k < n_steps; ++k) {
     uint64_t t = t0 + (uint64_t)k;
-    if (shared)
-      for (size_t kk = 0; kk < K; ++kk) sum[kk] = 0.0f;
     for (int i = 0; i < N; ++i) {
       size_t mo = c->map_mode == 1 ? 0 : (size_t)i * S;
       float u;
@@ -421,11 +546,10 @@ int orc_run(const orc_config* c, const uint8_t* cls, const float* cr, const int3
         tr_d[o] = done[i];
       }
     }
-    if (shared)
-      for (size_t kk = 0; kk < K; ++kk) Q[kk] = Q[kk] + sum[kk];
+    if (shared) tree_apply(sum, Q);
   }
   free(tab);
-  free(sum);
+  tree_free(&tree);
   return 0;
 }
 

@@ -64,6 +64,8 @@ class Oracle:
         lib.orc_td_update_one.restype = None
         lib.orc_td_update_batch.argtypes = [vp, C.c_int, C.c_int, C.c_int, vp, vp, vp, vp, vp, f32, f32,
                                             C.c_int]
+        lib.orc_tree_sum.argtypes = [vp, vp, C.c_int, C.c_int, vp]
+        lib.orc_tree_sum_bruteforce.argtypes = [vp, vp, C.c_int, C.c_int, vp]
         lib.orc_eps_table.argtypes = [vp, vp, C.c_int]
         lib.orc_run.argtypes = [vp, vp, vp, vp, vp, vp, vp, vp, vp, vp, vp, u64, i32, vp, vp, i32, vp, vp,
                                 vp, vp]
@@ -120,6 +122,14 @@ class Oracle:
         rc = self.lib.orc_td_update_batch(self._p(Q), S, A, s.size, self._p(s), self._p(a), self._p(r),
                                           self._p(s2), self._p(done), lr, gamma, mode)
         assert rc == 0
+
+    def tree_sum(self, key, d, K, brute=False):
+        key = np.ascontiguousarray(key, np.int32)
+        d = np.ascontiguousarray(d, np.float32)
+        out = np.empty(K, np.float32)
+        fn = self.lib.orc_tree_sum_bruteforce if brute else self.lib.orc_tree_sum
+        assert fn(self._p(key), self._p(d), key.size, K, self._p(out)) == 0
+        return out
 
     def eps_table(self, cfg):
         n = self.lib.orc_eps_table(C.byref(cfg), None, 0)

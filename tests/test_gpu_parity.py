@@ -83,6 +83,30 @@ def test_fused_chunked_equals_one_launch(gpu, oracle):
     run_both(gpu, oracle, cfg, cls, start, 101, chunks=[1, 1, 3, 7, 30, 59])
 
 
+def test_fused_result_independent_of_resident_envs(gpu, oracle):
+    """Few envs in flight (blocks loop over chunks, re-staging maps) == all at once."""
+    N, W, H, T = 3000, 16, 16, 150
+    cls, start = gpu.gen_maps_bernoulli(31, N, N, W, H, 0.1, 0.02)
+    cfg = gpu.make_config(N, W, H, episode_len=40, eps0=0.2, gamma=0.95, seed=17)
+    outs = []
+    for resident in (0, 64, 640, 1000):
+        with gpu.Engine(cfg, 0) as eng:
+            eng.set_maps(cls, start)
+            eng.set_resident_envs(resident)
+            if resident:
+                assert eng.fused_kernel_info()["grid"] == max(1, resident // eng.fused_kernel_info()["block"])
+            eng.set_trace(N, T)
+            eng.run_fused(T)
+            outs.append((eng.get_trace(T), eng.q_get(0, N), eng.get_state()))
+    Q = np.zeros((N, W * H, 4), np.float32)
+    st = oracle.new_state(cfg, start)
+    want = oracle.run(cfg, cls, None, start, Q, st, 0, T, trace_n=N)
+    for tr, q, got in outs:
+        assert_trace_equal(tr, want)
+        assert_q_close(q, Q)
+        assert np.array_equal(got["s"], st["s"]) and np.array_equal(got["episode"], st["episode"])
+
+
 def test_fused_large_map_global_path(gpu, oracle):
     """Maps too large for LDS are read from global memory (config 5 shape: 8
     actions, value-noise walls, per-cell rewards, linear epsilon)."""
@@ -228,6 +252,67 @@ def test_td_update_batch_matches_oracle(gpu, oracle, mode, n):
     want = Q0.copy().reshape(-1)
     oracle.td_update_batch(want, S, A, s, a, r, s2, done, 0.1, 0.99, mode)
     assert_q_close(got.reshape(-1), want)
+
+
+def _td_case(gpu, oracle, W, H, A, s, a, r, s2, done, mode=0):
+    S = W * H
+    cfg = gpu.make_config(1, W, H, n_actions=A, max_mode=mode, table_mode=gpu.TABLE_SHARED,
+                          map_mode=gpu.MAP_SHARED)
+    rng = np.random.default_rng(S)
+    Q0 = rng.normal(0, 1, (S, A)).astype(np.float32)
+    with gpu.Engine(cfg, 0) as eng:
+        eng.q_set(0, Q0)
+        eng.td_update(0, s, a, r, s2, done)
+        got = eng.q_get(0)
+    want = Q0.copy().reshape(-1)
+    oracle.td_update_batch(want, S, A, s, a, r, s2, done, 0.1, 0.99, mode)
+    assert_q_close(got.reshape(-1), want)
+
+
+def test_td_update_many_blocks_and_tiles(gpu, oracle):
+    """70 000 samples = 274 blocks: more than one 256-block tile and 18 groups;
+    deltas of mixed magnitude make a wrong association visible."""
+    W, H, A, n = 8, 8, 4, 70000
+    rng = np.random.default_rng(5)
+    S = W * H
+    s, a, s2 = rng.integers(0, S, n), rng.integers(0, A, n), rng.integers(0, S, n)
+    r = (rng.normal(0, 1, n) * 10.0 ** rng.integers(-3, 3, n)).astype(np.float32)
+    _td_case(gpu, oracle, W, H, A, s, a, r, s2, (rng.random(n) < 0.2).astype(np.uint8))
+
+
+def test_td_update_slot_overflow_path(gpu, oracle):
+    """One block holds 40 distinct keys of the same owner workgroup (more than a
+    block can hand over): the owner re-reads that block's samples in order."""
+    W, H, A = 64, 64, 4
+    owner, mix = 5, 37
+    keys = [(h << 8) | ((owner - mix * h) & 255) for h in range(40)]
+    rng = np.random.default_rng(9)
+    n = 3 * 256
+    key = rng.integers(0, W * H * A, n)
+    key[256:256 + 200] = rng.choice(keys, 200)  # block 1 overflows owner 5
+    s, a = key // A, key % A
+    s2 = rng.integers(0, W * H, n)
+    r = rng.normal(0, 1, n).astype(np.float32)
+    _td_case(gpu, oracle, W, H, A, s, a, r, s2, np.zeros(n, np.uint8))
+
+
+def test_td_update_large_table_scan_path(gpu, oracle):
+    """More than 16384 keys: the scanning fallback, same tree order."""
+    W, H, A, n = 80, 80, 8, 9000
+    rng = np.random.default_rng(3)
+    S = W * H
+    hot = rng.integers(0, S, 30)  # few cells: long runs per key across blocks and groups
+    s, a, s2 = rng.choice(hot, n), rng.integers(0, A, n), rng.integers(0, S, n)
+    r = (rng.normal(0, 1, n) * 10.0 ** rng.integers(-3, 3, n)).astype(np.float32)
+    _td_case(gpu, oracle, W, H, A, s, a, r, s2, (rng.random(n) < 0.1).astype(np.uint8), mode=1)
+
+
+def test_shared_table_large_table_scan_path(gpu, oracle):
+    N, W, H = 6000, 72, 72  # 20736 keys > 16384
+    cls, start = gpu.gen_maps_bernoulli(8, 1, N, W, H, 0.15)
+    cfg = gpu.make_config(N, W, H, table_mode=gpu.TABLE_SHARED, map_mode=gpu.MAP_SHARED, lr=0.01,
+                          eps0=0.2, seed=2)
+    run_both(gpu, oracle, cfg, cls, start, 40, trace_n=N)
 
 
 # ---- step rule, exhaustively, through the engine ------------------------------------

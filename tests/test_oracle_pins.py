@@ -304,12 +304,65 @@ def test_td_matches_float64_train_py(oracle):
     assert np.allclose(q32, ref, rtol=1e-5, atol=1e-6)
 
 
+def tree_sum_py(key, d, K):
+    """The ordered tree by its definition: blocks of 256 samples, groups of 16
+    blocks, each level added left to right from +0.0f."""
+    f = np.float32
+    total = np.zeros(K, np.float32)
+    n = len(key)
+    for k in range(K):
+        tot = f(0)
+        for g0 in range(0, n, 256 * 16):
+            gs = f(0)
+            for b0 in range(g0, min(n, g0 + 256 * 16), 256):
+                bs = f(0)
+                for i in range(b0, min(n, b0 + 256)):
+                    if key[i] == k:
+                        bs = f(bs + d[i])
+                gs = f(gs + bs)
+            tot = f(tot + gs)
+        total[k] = tot
+    return total
+
+
+def test_ordered_tree_sum(oracle):
+    """The touched-keys implementation == the definition, in C and in Python;
+    deltas of mixed magnitude make any other association visible."""
+    rng = np.random.default_rng(23)
+    for n, K in ((1, 4), (200, 8), (256, 3), (257, 3), (4096, 5), (4097, 5), (9000, 7), (70000, 6)):
+        key = rng.integers(-1, K, n).astype(np.int32)
+        d = (rng.normal(0, 1, n) * 10.0 ** rng.integers(-4, 4, n)).astype(np.float32)
+        fast = oracle.tree_sum(key, d, K)
+        assert np.array_equal(fast, oracle.tree_sum(key, d, K, brute=True)), (n, K)
+        if n <= 9000:
+            assert np.array_equal(fast, tree_sum_py(key, d, K)), (n, K)
+    # the order matters: one long run of a key is not summed left to right past a block edge
+    key = np.zeros(600, np.int32)
+    d = (rng.normal(0, 1, 600) * 10.0 ** rng.integers(-4, 4, 600)).astype(np.float32)
+    ltr = np.float32(0)
+    for v in d:
+        ltr = np.float32(ltr + v)
+    tree = oracle.tree_sum(key, d, 1)[0]
+    assert tree == tree_sum_py(key, d, 1)[0]
+    assert abs(float(tree) - float(ltr)) <= 1e-5 * abs(float(ltr)) + 1e-3  # same sum, other rounding
+    # up to 256 samples it IS left to right
+    assert oracle.tree_sum(key[:256], d[:256], 1)[0] == np.float32(sum_ltr(d[:256]))
+
+
+def sum_ltr(d):
+    acc = np.float32(0)
+    for v in d:
+        acc = np.float32(acc + v)
+    return acc
+
+
 def test_td_batch_rule_brute_force(oracle):
-    """Pre-batch reads, per-(s,a) sums in sample order from +0, then apply."""
+    """Pre-batch reads, per-(s,a) sums in sample order from +0, then apply
+    (n <= 256 here, where the tree is plain left-to-right summation)."""
     rng = np.random.default_rng(17)
     S, A, lr, gamma = 6, 4, np.float32(0.1), np.float32(0.99)
     for mode in (0, 1):
-        for n in (1, 5, 64, 300):
+        for n in (1, 5, 64, 256):
             Q = rng.normal(0, 1, S * A).astype(np.float32)
             s, a, s2 = rng.integers(0, S, n), rng.integers(0, A, n), rng.integers(0, S, n)
             r = rng.normal(0, 1, n).astype(np.float32)
@@ -439,7 +492,8 @@ def test_run_matches_python_loop(oracle, pycrl):
 
 
 def test_run_shared_table_order(oracle, pycrl):
-    """Shared table: per-(s,a) sums in env order from the pre-step table."""
+    """Shared table: per-(s,a) sums in env order from the pre-step table (64
+    envs: one block, so the tree is left-to-right; larger N in the next test)."""
     W, H, A, N = 4, 4, 4, 64
     cls, start = pycrl.gen_maps_bernoulli(1, 1, N, W, H, 0.1)
     cfg = pycrl.make_config(N, W, H, table_mode=pycrl.TABLE_SHARED, map_mode=pycrl.MAP_SHARED, eps0=0.5,
@@ -464,4 +518,29 @@ def test_run_shared_table_order(oracle, pycrl):
             acc = np.float32(acc + d)
         want[k] = np.float32(pre[k] + acc)
     assert max(len(v) for v in lists.values()) > 1  # collisions exist
+    assert np.array_equal(Q, want)
+
+
+def test_run_shared_table_uses_the_tree(oracle, pycrl):
+    """N > 256: one shared-table step == deltas from the pre-step table pushed
+    through the block/group tree."""
+    W, H, A, N = 5, 5, 4, 9000
+    cls, start = pycrl.gen_maps_bernoulli(2, 1, N, W, H, 0.1)
+    cfg = pycrl.make_config(N, W, H, table_mode=pycrl.TABLE_SHARED, map_mode=pycrl.MAP_SHARED, eps0=0.5,
+                            lr=0.001, seed=4)
+    rng = np.random.default_rng(1)
+    Q = rng.normal(0, 0.1, W * H * A).astype(np.float32)
+    pre = Q.copy()
+    st = oracle.new_state(cfg, start)
+    s_before = st["s"].copy()
+    tr = oracle.run(cfg, cls, None, start, Q, st, 0, 1, trace_n=N)
+    f = np.float32
+    key = s_before.astype(np.int64) * A + tr["action"][0]
+    d = np.empty(N, np.float32)
+    for i in range(N):
+        s2 = int(tr["s_next"][0, i])
+        m = f(0) if tr["done"][0, i] else pre[s2 * A:(s2 + 1) * A].max()
+        target = f(np.float64(f(0.99)) * np.float64(m) + np.float64(tr["reward"][0, i]))
+        d[i] = f(f(0.001) * f(target - pre[key[i]]))
+    want = (pre + oracle.tree_sum(key, d, W * H * A)).astype(np.float32)
     assert np.array_equal(Q, want)
