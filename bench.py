@@ -229,8 +229,9 @@ def main():
 
     if not args.no_cpu:
         threads = min(16, os.cpu_count() or 1)
-        n_sample = {"c2": 4096, "c3": 65536, "c4": 1 << 18, "c5": 256}[key]
-        cpu_steps = {"c2": 50000, "c3": 100, "c4": 1000, "c5": 8192}[key]
+        # about 10-30 s of CPU work each (the wall time is that divided by the threads)
+        n_sample = {"c2": 4096, "c3": 65536, "c4": 1 << 18, "c5": 2048}[key]
+        cpu_steps = {"c2": 50000, "c3": 1500, "c4": 1000, "c5": 16384}[key]
         v, cores, dt = time_cpu(key, min(n_sample, g["n"]), cpu_steps, threads)
         out["cpu_baseline"] = {"value": v, "unit": "env-steps/s", "cores": cores, "kind": "port",
                                "sample": "%d envs x %d steps of the same workload, %.1f s wall on %d threads"

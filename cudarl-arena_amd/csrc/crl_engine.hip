@@ -92,7 +92,6 @@ struct crl_engine {
   DevBuf<int32_t> key;
   DevBuf<float> delta;
   DevBuf<uint2> handoff;
-  DevBuf<uint8_t> handoff_count;
   bool lds_opt_in = false;
   // scratch of crl_td_update
   DevBuf<int32_t> b_s, b_a, b_s2;
@@ -249,7 +248,8 @@ void launch_fused_a(const crl_engine* e, const FusedPlan& p, uint64_t t0, int n)
   }
 }
 
-constexpr size_t kHandoffLimitBytes = (size_t)64 << 20;
+constexpr size_t kHandoffLimitBytes = (size_t)128 << 20;
+constexpr size_t kLdsPerWorkgroup = 160 * 1024;  // gfx950
 
 int ceil_log2(size_t v) {
   int b = 0;
@@ -267,7 +267,7 @@ crl::ReduceGeom reduce_geom(const crl_engine* e, int n) {
 }
 
 size_t handoff_records(const crl::ReduceGeom& G) {
-  return ((size_t)1 << G.own_shift) * (size_t)G.n_blocks * crl::kSlotCap;
+  return ((size_t)1 << G.own_shift) * (size_t)G.n_blocks * crl::kHandoffRecs;
 }
 
 // the two-pass reduction needs the dense LDS table (K <= 16384) and a bounded hand-off buffer
@@ -287,7 +287,7 @@ hipError_t allow_lds(Kern kern, size_t bytes) {
 // kernels that use more than the default 64 KB of LDS per workgroup (gfx950 has 160 KB)
 int opt_in_lds(crl_engine* e) {
   if (e->lds_opt_in) return CRL_OK;
-  const size_t act = sizeof(crl::ReduceLds) + (size_t)kLdsMapLimitBytes;
+  const size_t act = kLdsPerWorkgroup;  // what a launch asks for is checked against this
   HIP_TRY(allow_lds(crl::k_reduce_blocks, sizeof(crl::ReduceLds)));
   HIP_TRY(allow_lds(crl::k_reduce_owners, kOwnersLds));
   HIP_TRY(allow_lds(crl::k_shared_act<4, 1, true>, act));
@@ -301,7 +301,6 @@ int opt_in_lds(crl_engine* e) {
 int ensure_handoff(crl_engine* e, const crl::ReduceGeom& G) {
   const size_t recs = handoff_records(G);
   hipError_t h = e->handoff.ensure(recs);
-  if (h == hipSuccess) h = e->handoff_count.ensure(recs / crl::kSlotCap);
   if (h != hipSuccess) return fail(CRL_E_ALLOC, "hand-off buffer allocation failed: %s", hipGetErrorString(h));
   return opt_in_lds(e);
 }
@@ -309,7 +308,7 @@ int ensure_handoff(crl_engine* e, const crl::ReduceGeom& G) {
 int reduce_owners(crl_engine* e, const crl::ReduceGeom& G, float* Q, const int32_t* key,
                   const float* delta, int n) {
   hipLaunchKernelGGL(crl::k_reduce_owners, dim3(1 << G.own_shift), dim3(256), kOwnersLds, e->stream, G,
-                     Q, key, delta, n, e->handoff.p, e->handoff_count.p);
+                     Q, key, delta, n, e->handoff.p);
   HIP_TRY(hipGetLastError());
   return CRL_OK;
 }
@@ -327,8 +326,7 @@ int reduce_apply(crl_engine* e, float* Q, const int32_t* key, const float* delta
   int rc = ensure_handoff(e, G);
   if (rc) return rc;
   hipLaunchKernelGGL(crl::k_reduce_blocks, dim3(G.n_blocks), dim3(crl::kBlockSamples),
-                     sizeof(crl::ReduceLds), e->stream, G, key, delta, n, e->handoff.p,
-                     e->handoff_count.p);
+                     sizeof(crl::ReduceLds), e->stream, G, key, delta, n, e->handoff.p);
   HIP_TRY(hipGetLastError());
   return reduce_owners(e, G, Q, key, delta, n);
 }
@@ -338,14 +336,13 @@ void launch_shared_act(crl_engine* e, bool reduce, const crl::ReduceGeom& G, uin
   const crl::Rules R = e->rules();
   const crl::Ptrs P = e->ptrs();
   const int block = 256, grid = (e->N + block - 1) / block;
-  const size_t map_lds = MAP == 1 ? (size_t)e->map_words * 4 : 0;
+  const size_t lds = (reduce ? sizeof(crl::ReduceLds) : 0) + (MAP == 1 ? (size_t)e->map_words * 4 : 0);
   if (reduce)
-    hipLaunchKernelGGL((crl::k_shared_act<A, MAP, true>), dim3(grid), dim3(block),
-                       sizeof(crl::ReduceLds) + map_lds, e->stream, R, P, t, trace_row, e->key.p,
-                       e->delta.p, G, e->handoff.p, e->handoff_count.p);
+    hipLaunchKernelGGL((crl::k_shared_act<A, MAP, true>), dim3(grid), dim3(block), lds, e->stream, R, P,
+                       t, trace_row, e->key.p, e->delta.p, G, e->handoff.p);
   else
-    hipLaunchKernelGGL((crl::k_shared_act<A, MAP, false>), dim3(grid), dim3(block), map_lds, e->stream,
-                       R, P, t, trace_row, e->key.p, e->delta.p, G, e->handoff.p, e->handoff_count.p);
+    hipLaunchKernelGGL((crl::k_shared_act<A, MAP, false>), dim3(grid), dim3(block), lds, e->stream, R,
+                       P, t, trace_row, e->key.p, e->delta.p, G, e->handoff.p);
 }
 
 // one shared-table step: act (select + move + delta + block sums), then the key owners
@@ -356,8 +353,15 @@ int shared_step(crl_engine* e, uint64_t t, int trace_row) {
     int rc = ensure_handoff(e, G);
     if (rc) return rc;
   }
-  const bool lds_map =
-      e->cfg.map_mode == CRL_MAP_SHARED && (size_t)e->map_words * 4 <= (size_t)kLdsMapLimitBytes;
+  // LDS plan of the act kernel: reduction table (fast path), then the map.  The
+  // shared table itself stays in L2: streaming its 64 KB into every workgroup's
+  // LDS each step measured slower than the two row reads it saves.
+  size_t lds = fast ? sizeof(crl::ReduceLds) : 0;
+  const size_t limit = fast ? kLdsPerWorkgroup : (size_t)64 * 1024;
+  const size_t map_bytes = (size_t)e->map_words * 4;
+  const bool lds_map = e->cfg.map_mode == CRL_MAP_SHARED && map_bytes <= (size_t)kLdsMapLimitBytes &&
+                       lds + map_bytes <= limit;
+  if (lds_map) lds += map_bytes;
   if (e->A == 4) {
     if (lds_map) launch_shared_act<4, 1>(e, fast, G, t, trace_row);
     else launch_shared_act<4, 2>(e, fast, G, t, trace_row);

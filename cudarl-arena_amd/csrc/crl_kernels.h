@@ -352,17 +352,18 @@ __global__ __launch_bounds__(256) void k_shared_act(const Rules R, const Ptrs P,
                                                      const int trace_row,
                                                      int32_t* __restrict__ key,
                                                      float* __restrict__ delta, const ReduceGeom G,
-                                                     uint2* __restrict__ handoff,
-                                                     uint8_t* __restrict__ handoff_count) {
+                                                     uint2* __restrict__ handoff) {
   extern __shared__ unsigned char lds_raw[];
   uint32_t* lds_map = reinterpret_cast<uint32_t*>(lds_raw + (REDUCE ? sizeof(ReduceLds) : 0));
   const int tid = threadIdx.x;
   const int env = blockIdx.x * blockDim.x + tid;
+  const bool live = env < P.N;
+  // the env's cell is fetched while the map streams into LDS
+  const int s_in = live ? P.s[env] : 0;
   if (MAP == 1) {
     for (int i = tid; i < P.map_words; i += blockDim.x) lds_map[i] = P.map[i];
     __syncthreads();
   }
-  const bool live = env < P.N;
   int my_key = 0;
   float my_delta = 0.0f;
   if (live) {
@@ -375,7 +376,7 @@ __global__ __launch_bounds__(256) void k_shared_act(const Rules R, const Ptrs P,
         P.cell_reward ? P.cell_reward + (P.map_shared ? 0 : (size_t)env * P.S) : nullptr;
     const float* __restrict__ Q = P.Q;
 
-    const int s0 = P.s[env];
+    const int s0 = s_in;
     int x = s0 % R.W, y = s0 / R.W;
     const Row<A> row = load_row<A>(Q + (size_t)s0 * A);
     Draw d = pick_draw(explore_block(R.seed, (uint32_t)env, t >> 1), t, A);
@@ -421,7 +422,7 @@ __global__ __launch_bounds__(256) void k_shared_act(const Rules R, const Ptrs P,
   }
   if (REDUCE) {
     ReduceLds& L = *reinterpret_cast<ReduceLds*>(lds_raw);
-    reduce_block(L, G, blockIdx.x, my_key, my_delta, live, handoff, handoff_count);
+    reduce_block(L, G, blockIdx.x, my_key, my_delta, live, handoff);
   }
 }
 

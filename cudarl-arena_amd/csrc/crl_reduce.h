@@ -24,7 +24,8 @@ namespace crl {
 constexpr int kBlockSamples = 256;   // level 0
 constexpr int kGroupBlocks = 16;     // level 1
 constexpr int kOwnKeys = 64;         // keys per owner workgroup
-constexpr int kSlotCap = 8;          // block sums one block can hand one owner
+constexpr int kSlotCap = 15;         // block sums one block can hand one owner
+constexpr int kHandoffRecs = 16;     // one 128-byte hand-off cell: header {count, -} + 15 records
 constexpr int kSlotOverflow = 255;   // count value: read the block's raw samples instead
 constexpr int kDenseKeys = 16384;    // keys the dense LDS table of pass 1 can hold
 constexpr int kTileBlocks = 256;     // blocks per LDS tile of pass 2
@@ -60,8 +61,7 @@ struct ReduceLds {
 // sample (valid = false: no sample / no delta).  key < K <= kDenseKeys.
 __device__ __forceinline__ void reduce_block(ReduceLds& L, const ReduceGeom G, const int block,
                                              const int key, const float delta, const bool valid,
-                                             uint2* __restrict__ handoff,
-                                             uint8_t* __restrict__ handoff_count) {
+                                             uint2* __restrict__ handoff) {
   const int tid = threadIdx.x;
   const int lane = tid & 63;
   const int wave = tid >> 6;
@@ -108,13 +108,16 @@ __device__ __forceinline__ void reduce_block(ReduceLds& L, const ReduceGeom G, c
     __syncthreads();
   }
 
+  // hand-off cell of (owner, block): record 0 is the header, so that the owner
+  // gets count and records with one independent 128-byte read
   if (leader && first && slot < kSlotCap) {
-    const size_t at = ((size_t)owner * G.n_blocks + block) * kSlotCap + slot;
+    const size_t at = ((size_t)owner * G.n_blocks + block) * kHandoffRecs + 1 + slot;
     handoff[at] = make_uint2((uint32_t)(key >> G.own_shift), __float_as_uint(L.run[key]));
   }
   if (tid < n_own) {
     const int c = L.handed[tid];
-    handoff_count[(size_t)tid * G.n_blocks + block] = (uint8_t)(c > kSlotCap ? kSlotOverflow : c);
+    handoff[((size_t)tid * G.n_blocks + block) * kHandoffRecs] =
+        make_uint2((uint32_t)(c > kSlotCap ? kSlotOverflow : c), 0u);
   }
 }
 
@@ -123,23 +126,21 @@ __global__ __launch_bounds__(kBlockSamples) void k_reduce_blocks(const ReduceGeo
                                                                  const int32_t* __restrict__ key,
                                                                  const float* __restrict__ delta,
                                                                  const int n,
-                                                                 uint2* __restrict__ handoff,
-                                                                 uint8_t* __restrict__ handoff_count) {
+                                                                 uint2* __restrict__ handoff) {
   extern __shared__ unsigned char lds_raw[];
   ReduceLds& L = *reinterpret_cast<ReduceLds*>(lds_raw);
   const int i = blockIdx.x * kBlockSamples + threadIdx.x;
   const int k = i < n ? key[i] : -1;
   const bool valid = k >= 0;
   const float d = valid ? delta[i] : 0.0f;
-  reduce_block(L, G, blockIdx.x, valid ? k : 0, d, valid, handoff, handoff_count);
+  reduce_block(L, G, blockIdx.x, valid ? k : 0, d, valid, handoff);
 }
 
 // Pass 2: one workgroup per owner (64 keys).
 __global__ __launch_bounds__(256) void k_reduce_owners(const ReduceGeom G, float* __restrict__ Q,
                                                         const int32_t* __restrict__ key,
                                                         const float* __restrict__ delta, const int n,
-                                                        const uint2* __restrict__ handoff,
-                                                        const uint8_t* __restrict__ handoff_count) {
+                                                        const uint2* __restrict__ handoff) {
   extern __shared__ float tile[];  // [kTileBlocks][64] block sums, then [16][64] group sums
   float* gsum = tile + kTileBlocks * kOwnKeys;
   const int tid = threadIdx.x;
@@ -147,29 +148,42 @@ __global__ __launch_bounds__(256) void k_reduce_owners(const ReduceGeom G, float
   const int wave = tid >> 6;
   const int owner = blockIdx.x;
   float total = 0.0f;
+  // the table entry this lane will update: fetched now, needed last
+  const int my_key = key_of(owner, lane, G.own_shift);
+  const float q_old = (wave == 0 && my_key < G.K) ? Q[my_key] : 0.0f;
 
   for (int b0 = 0; b0 < G.n_blocks; b0 += kTileBlocks) {
+    const int b = b0 + tid;
+    // the whole hand-off cell in one go: no load depends on another
+    uint4 cell[kHandoffRecs / 2];
+    if (b < G.n_blocks) {
+      const uint4* src = reinterpret_cast<const uint4*>(handoff + ((size_t)owner * G.n_blocks + b) * kHandoffRecs);
+#pragma unroll
+      for (int i = 0; i < kHandoffRecs / 2; ++i) cell[i] = src[i];
+    } else {
+#pragma unroll
+      for (int i = 0; i < kHandoffRecs / 2; ++i) cell[i] = make_uint4(0, 0, 0, 0);
+    }
     float4* my_row = reinterpret_cast<float4*>(tile + tid * kOwnKeys);
 #pragma unroll
     for (int i = 0; i < kOwnKeys / 4; ++i) my_row[i] = make_float4(0.0f, 0.0f, 0.0f, 0.0f);
-    const int b = b0 + tid;
-    if (b < G.n_blocks) {
-      const int c = handoff_count[(size_t)owner * G.n_blocks + b];
-      if (c != kSlotOverflow) {
-        const uint2* rec = handoff + ((size_t)owner * G.n_blocks + b) * kSlotCap;
-        for (int i = 0; i < c; ++i) {
-          const uint2 r = rec[i];
-          tile[tid * kOwnKeys + r.x] = __uint_as_float(r.y);
-        }
-      } else {
-        // more distinct keys than slots: redo the block's part from its samples, in order
-        const int lo = b * kBlockSamples, hi = min(n, lo + kBlockSamples);
-        for (int i = lo; i < hi; ++i) {
-          const int k = key[i];
-          if (k >= 0 && owner_of(k, G.own_shift) == owner) {
-            float& cell = tile[tid * kOwnKeys + (k >> G.own_shift)];
-            cell = cell + delta[i];
-          }
+    const int c = (int)cell[0].x;
+    if (c != kSlotOverflow) {
+      float* row = tile + tid * kOwnKeys;
+      if (c > 0) row[cell[0].z] = __uint_as_float(cell[0].w);
+#pragma unroll
+      for (int i = 1; i < kHandoffRecs / 2; ++i) {
+        if (c > 2 * i - 1) row[cell[i].x] = __uint_as_float(cell[i].y);
+        if (c > 2 * i) row[cell[i].z] = __uint_as_float(cell[i].w);
+      }
+    } else {
+      // more distinct keys than slots: redo the block's part from its samples, in order
+      const int lo = b * kBlockSamples, hi = min(n, lo + kBlockSamples);
+      for (int i = lo; i < hi; ++i) {
+        const int k = key[i];
+        if (k >= 0 && owner_of(k, G.own_shift) == owner) {
+          float& acc = tile[tid * kOwnKeys + (k >> G.own_shift)];
+          acc = acc + delta[i];
         }
       }
     }
@@ -190,10 +204,7 @@ __global__ __launch_bounds__(256) void k_reduce_owners(const ReduceGeom G, float
     }
     __syncthreads();
   }
-  if (wave == 0) {
-    const int k = key_of(owner, lane, G.own_shift);
-    if (k < G.K) Q[k] = Q[k] + total;
-  }
+  if (wave == 0 && my_key < G.K) Q[my_key] = q_old + total;
 }
 
 // Fallback for tables with more than kDenseKeys keys (or too many blocks for the
