@@ -36,7 +36,9 @@ WORKLOADS = {
                name="c2: 4096 envs 32x32, per-env tables 1024x4, eps 0.1, T=256"),
     "c3": dict(n=65536, w=64, h=64, a=4, t=0, steps=1000, warmup=50, bytes=24.0,
                name="c3: 65536 envs, shared 64x64 map, one shared table 4096x4, ordered reduction"),
-    "c4": dict(n=1 << 20, w=16, h=16, a=4, t=128, steps=1000, warmup=128, bytes=42.25,
+    # traffic: HBM bytes per env-step from rocprofv3 FETCH_SIZE x2.000 + WRITE_SIZE x1.000
+    # (profiles/k_fused_per_env_c4.md), valid for the default launch only
+    "c4": dict(n=1 << 20, w=16, h=16, a=4, t=128, steps=1000, warmup=128, bytes=42.25, traffic=48.2,
                name="c4: 1048576 envs 16x16, per-env tables 256x4 (4 GB), traps, eps 0.1, T=128"),
     "c5": dict(n=8192, w=256, h=256, a=8, t=1024, steps=1024, warmup=64, bytes=70.0,
                name="c5: 8192 envs 256x256, 8 actions, per-env tables 65536x8 (16 GB), cell rewards"),
@@ -223,9 +225,10 @@ def main():
                      "kernel_ms_per_launch": g["device_ms"] / args.launches,
                      "whole_job_GBps": achieved},
     }
-    traffic = os.environ.get("CRL_BENCH_TRAFFIC_BYTES")  # filled in from a rocprofv3 --pmc run
-    if traffic:
-        out["roofline"]["traffic"] = float(traffic)
+    if ("traffic" in wl and steps == wl["steps"] and args.launches == 1 and not args.envs
+            and not args.resident):
+        # measured in separate rocprofv3 --pmc runs of this same command, not in this run
+        out["roofline"]["traffic"] = wl["traffic"] * g["n"] * steps
 
     if not args.no_cpu:
         threads = min(16, os.cpu_count() or 1)
