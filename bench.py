@@ -97,7 +97,7 @@ class HipEvents:
         return float(ms.value)
 
 
-def time_gpu(key, steps, warmup, launches=1, n_override=None, resident=0):
+def time_gpu(key, steps, warmup, launches=1, n_override=None, resident=0, variant=0):
     """-> dict(steps_per_s, ms_per_step, kernel_ms, wall_s, info)"""
     wl = WORKLOADS[key]
     cfg, cls, start, cr = build_workload(key, n_override)
@@ -108,6 +108,8 @@ def time_gpu(key, steps, warmup, launches=1, n_override=None, resident=0):
         del cls, cr
         if resident:
             eng.set_resident_envs(resident)
+        if variant:
+            eng.set_fused_variant(variant)
         info = eng.fused_kernel_info()
         if warmup:
             eng.run_fused(warmup)
@@ -125,9 +127,10 @@ def time_gpu(key, steps, warmup, launches=1, n_override=None, resident=0):
         wall = time.perf_counter() - t0
         dev_ms = ev.elapsed_ms(a, b)
         st = eng.get_state()
+        split = eng.fused_split()
     secs = max(wall, dev_ms * 1e-3)
     return dict(n=n, steps_per_s=n * steps / secs, ms_per_step=secs * 1e3 / steps, device_ms=dev_ms,
-                wall_s=wall, launches=launches, info=info, episodes_min=int(st["episode"].min()),
+                wall_s=wall, launches=launches, info=info, split=split, episodes_min=int(st["episode"].min()),
                 bytes_per_step=wl["bytes"])
 
 
@@ -178,6 +181,7 @@ def main():
     ap.add_argument("--launches", type=int, default=1, help="split the K timed steps over this many launches")
     ap.add_argument("--envs", type=int, default=None, help="override the env count (not a headline figure)")
     ap.add_argument("--resident", type=int, default=0, help="envs in flight at once (0 = automatic)")
+    ap.add_argument("--variant", type=int, default=0, help="fused kernel: 0 automatic, 1 plain, 2 hybrid")
     ap.add_argument("--probe-copy", type=int, default=0, metavar="MIB",
                     help="only run one plain copy kernel of this many MiB (calibrates rocprofv3 counters)")
     ap.add_argument("--no-cpu", action="store_true", help="skip the cpu_baseline leg")
@@ -198,7 +202,7 @@ def main():
     wl = WORKLOADS[key]
     steps = args.steps if args.steps is not None else wl["steps"]
     warmup = args.warmup if args.warmup is not None else wl["warmup"]
-    g = time_gpu(key, steps, warmup, args.launches, args.envs, args.resident)
+    g = time_gpu(key, steps, warmup, args.launches, args.envs, args.resident, args.variant)
 
     achieved = g["steps_per_s"] * wl["bytes"] / 1e9
     # the dominant kernel's own duration (device events around its launches)
@@ -218,7 +222,8 @@ def main():
         "data": "synthetic (Philox-seeded maps, zero-initialised tables)",
         "config": {"workload": wl["name"], "n_envs": g["n"], "steps_per_launch": steps // args.launches,
                    "kernel": g["info"]["name"], "grid": g["info"]["grid"], "block": g["info"]["block"],
-                   "lds_bytes": g["info"]["lds_bytes"]},
+                   "lds_bytes": g["info"]["lds_bytes"],
+                   "envs_stepped_from_hbm_tables": g["split"][0], "envs_stepped_from_lds_tables": g["split"][1]},
         "roofline": {"bound": "hbm", "achieved": kern_achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s",
                      "frac": kern_achieved / HBM_PEAK_GBS, "traffic": None,
                      "algorithmic_bytes_per_env_step": wl["bytes"],

@@ -73,6 +73,9 @@ struct crl_engine {
   int n_maps = 0, n_tables = 0, map_words = 0;
   uint64_t t = 0;
   long resident_envs = 0;  // 0 = automatic
+  int fused_variant = 0;   // 0 = automatic, 1 = plain, 2 = hybrid (when it fits)
+  DevBuf<unsigned> ticket;
+  bool hybrid_opt_in = false;
 
   DevBuf<int32_t> s, ep_step, episode, start, act;
   DevBuf<float> reward;
@@ -186,7 +189,14 @@ struct FusedPlan {
   int block, grid;
   size_t lds;
   const char* name;
+  bool tickets;    // per-env maps in LDS: waves draw env ranges from a ticket counter
+  bool hybrid;     // ... with a fifth wave per workgroup that steps envs whose tables it holds in LDS
+  bool fast;       // the folded loop for the common configuration
+  int tab_stride;  // floats between two tables in LDS
 };
+
+constexpr size_t kLdsPerWorkgroup = 160 * 1024;  // gfx950
+constexpr int kHybridMinEnvs = 2048;
 
 FusedPlan plan_fused(const crl_engine* e) {
   FusedPlan p{};
@@ -208,11 +218,10 @@ FusedPlan plan_fused(const crl_engine* e) {
       p.map_kind = 2;
     }
   }
-  p.grid = (e->N + p.block - 1) / p.block;
-  // Envs live on the chip at once.  A block works through its chunks one after
-  // the other, so a smaller grid means fewer tables in flight: when all tables
-  // together exceed the last-level cache, keep as many in flight as fit into
-  // it (but never less than one wave per SIMD of the whole chip).
+  // Envs live on the chip at once.  A worker steps its envs for all n steps
+  // before it takes the next ones, so a smaller grid means fewer tables in
+  // flight: when all tables together exceed the last-level cache, keep as many
+  // in flight as fit into it (but never less than one wave per SIMD of the chip).
   long resident = e->resident_envs;
   if (resident <= 0) {
     const size_t table_bytes = e->K * sizeof(float);
@@ -220,11 +229,38 @@ FusedPlan plan_fused(const crl_engine* e) {
     if ((size_t)e->N * table_bytes > kLastLevelCacheBytes)
       resident = std::max<long>(kLanesOneWavePerSimd, (long)(kLastLevelCacheBytes / table_bytes));
   }
-  p.grid = (int)std::min<long>(p.grid, std::max<long>(1, resident / p.block));
+  p.tickets = p.map_kind == 0;
+  if (!p.tickets) {
+    p.grid = (int)std::min<long>((e->N + p.block - 1) / p.block, std::max<long>(1, resident / p.block));
+  } else {
+    const crl_config& c = e->cfg;
+    p.fast = c.eps_mode == CRL_EPS_FIXED && c.reward_flags == 0 && c.goal_mode == CRL_GOAL_ON_TARGET &&
+             c.auto_reset == 1 && c.max_mode == CRL_MAX_TRUE && e->trace_n == 0 && e->sup_n == 0;
+    // Hybrid workgroups when 32 whole tables (padded by one row against bank
+    // conflicts) and five waves' maps fit into LDS.
+    p.tab_stride = (int)e->K + 4;
+    const size_t map_lds = (size_t)e->map_words * 64 * 4;
+    const size_t hybrid_lds = 5 * map_lds + (size_t)crl::kTicketEnvs * p.tab_stride * 4;
+    const bool fits = e->K % 4 == 0 && hybrid_lds <= kLdsPerWorkgroup;
+    p.hybrid = fits && (e->fused_variant == 2 || (e->fused_variant == 0 && e->N >= kHybridMinEnvs));
+    p.block = p.hybrid ? 320 : 256;
+    p.lds = p.hybrid ? hybrid_lds : 4 * map_lds;
+    const long tickets = (e->N + crl::kTicketEnvs - 1) / crl::kTicketEnvs;
+    const long per_wg = p.hybrid ? 9 : 8;  // tickets one workgroup takes per round
+    p.grid = (int)std::min<long>(std::max<long>(1, resident / 256), (tickets + per_wg - 1) / per_wg);
+  }
   static const char* names[2][3] = {
       {"k_fused_per_env<4,0>", "k_fused_per_env<4,1>", "k_fused_per_env<4,2>"},
       {"k_fused_per_env<8,0>", "k_fused_per_env<8,1>", "k_fused_per_env<8,2>"}};
   p.name = names[e->A == 8][p.map_kind];
+  if (p.tickets) {
+    static const char* tnames[2][2][2] = {
+        {{"k_fused_tickets<4,general,hbm>", "k_fused_tickets<4,general,hbm+lds>"},
+         {"k_fused_tickets<4,fast,hbm>", "k_fused_tickets<4,fast,hbm+lds>"}},
+        {{"k_fused_tickets<8,general,hbm>", "k_fused_tickets<8,general,hbm+lds>"},
+         {"k_fused_tickets<8,fast,hbm>", "k_fused_tickets<8,fast,hbm+lds>"}}};
+    p.name = tnames[e->A == 8][p.fast][p.hybrid];
+  }
   return p;
 }
 
@@ -232,11 +268,21 @@ template <int A>
 void launch_fused_a(const crl_engine* e, const FusedPlan& p, uint64_t t0, int n) {
   const crl::Rules R = e->rules();
   const crl::Ptrs P = e->ptrs();
+  if (p.tickets) {
+    hipLaunchKernelGGL(crl::k_fill_u32, dim3(1), dim3(64), 0, e->stream, e->ticket.p, 0u, 3);
+    const dim3 g(p.grid), b(p.block);
+    unsigned* tk = e->ticket.p;
+    if (p.fast && p.hybrid)
+      hipLaunchKernelGGL((crl::k_fused_tickets<A, true, true>), g, b, p.lds, e->stream, R, P, t0, n, tk, p.tab_stride);
+    else if (p.fast)
+      hipLaunchKernelGGL((crl::k_fused_tickets<A, true, false>), g, b, p.lds, e->stream, R, P, t0, n, tk, p.tab_stride);
+    else if (p.hybrid)
+      hipLaunchKernelGGL((crl::k_fused_tickets<A, false, true>), g, b, p.lds, e->stream, R, P, t0, n, tk, p.tab_stride);
+    else
+      hipLaunchKernelGGL((crl::k_fused_tickets<A, false, false>), g, b, p.lds, e->stream, R, P, t0, n, tk, p.tab_stride);
+    return;
+  }
   switch (p.map_kind) {
-    case 0:
-      hipLaunchKernelGGL((crl::k_fused_per_env<A, 0>), dim3(p.grid), dim3(p.block), p.lds, e->stream,
-                         R, P, t0, n);
-      break;
     case 1:
       hipLaunchKernelGGL((crl::k_fused_per_env<A, 1>), dim3(p.grid), dim3(p.block), p.lds, e->stream,
                          R, P, t0, n);
@@ -249,7 +295,6 @@ void launch_fused_a(const crl_engine* e, const FusedPlan& p, uint64_t t0, int n)
 }
 
 constexpr size_t kHandoffLimitBytes = (size_t)128 << 20;
-constexpr size_t kLdsPerWorkgroup = 160 * 1024;  // gfx950
 
 int ceil_log2(size_t v) {
   int b = 0;
@@ -533,6 +578,26 @@ int crl_set_resident_envs(crl_engine* e, int32_t n_envs) {
   return CRL_OK;
 }
 
+int crl_set_fused_variant(crl_engine* e, int32_t variant) {
+  if (!e) return fail(CRL_E_ARG, "null engine");
+  if (variant < 0 || variant > 2) return fail(CRL_E_ARG, "variant must be 0 (automatic), 1 (plain) or 2 (hybrid)");
+  e->fused_variant = variant;
+  return CRL_OK;
+}
+
+int crl_get_fused_split(crl_engine* e, uint32_t* hbm_envs, uint32_t* lds_envs) {
+  int rc = check_engine(e);
+  if (rc) return rc;
+  unsigned v[3] = {0, 0, 0};
+  if (e->ticket.p) {
+    HIP_TRY(hipMemcpyAsync(v, e->ticket.p, sizeof v, hipMemcpyDeviceToHost, e->stream));
+    HIP_TRY(hipStreamSynchronize(e->stream));
+  }
+  if (hbm_envs) *hbm_envs = v[1];
+  if (lds_envs) *lds_envs = v[2];
+  return CRL_OK;
+}
+
 int crl_sync(crl_engine* e) {
   int rc = check_engine(e);
   if (rc) return rc;
@@ -726,6 +791,19 @@ int crl_run_fused(crl_engine* e, int32_t n_steps) {
   if (n_steps == 0) return CRL_OK;
   if (e->cfg.table_mode == CRL_TABLE_PER_ENV) {
     const FusedPlan p = plan_fused(e);
+    if (p.tickets) {
+      if (e->ticket.ensure(3) != hipSuccess) return fail(CRL_E_ALLOC, "ticket counter allocation failed");
+      if (!e->hybrid_opt_in) {
+        const void* fns[] = {
+            reinterpret_cast<const void*>(&crl::k_fused_tickets<4, true, true>),
+            reinterpret_cast<const void*>(&crl::k_fused_tickets<4, false, true>),
+            reinterpret_cast<const void*>(&crl::k_fused_tickets<8, true, true>),
+            reinterpret_cast<const void*>(&crl::k_fused_tickets<8, false, true>)};
+        for (const void* fn : fns)
+          HIP_TRY(hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, (int)kLdsPerWorkgroup));
+        e->hybrid_opt_in = true;
+      }
+    }
     if (e->A == 4)
       launch_fused_a<4>(e, p, e->t, n_steps);
     else

@@ -64,14 +64,184 @@ __device__ __forceinline__ Draw pick_draw(const Philox4 blk, uint64_t t, int A) 
 // ---------------------------------------------------------------------------
 // Fused select -> step -> update, per-env tables, one lane per env, n_steps per
 // launch.  The env's position, episode counters and the Q row of the cell it
-// stands on live in registers for the whole launch: per step the only memory
+// stands on live in registers for the whole launch: per step the only table
 // traffic is one row read (the new cell) and one 4-byte write.
-//
-// MAP = 0: per-env maps staged once into LDS, word-interleaved across lanes
-//          (word w of lane l at lds[w*blockDim + l]: conflict-free reads)
-// MAP = 1: one shared map staged into LDS
-// MAP = 2: maps read from global memory (too large for LDS)
 // ---------------------------------------------------------------------------
+
+// where an env's table lives while it is being stepped
+template <int A>
+struct GlobalTable {  // in HBM / the caches
+  float* __restrict__ q;
+  __device__ __forceinline__ Row<A> load(int s) const { return load_row<A>(q + (size_t)s * A); }
+  __device__ __forceinline__ void store(int s, int a, float v) const { q[(size_t)s * A + a] = v; }
+};
+template <int A>
+struct LdsTable {  // staged into LDS for the whole launch
+  float* q;
+  __device__ __forceinline__ Row<A> load(int s) const { return load_row<A>(q + s * A); }
+  __device__ __forceinline__ void store(int s, int a, float v) const { q[s * A + a] = v; }
+};
+
+// n_steps of one env.  `cls(cell)` gives the class of a cell of the env's map,
+// `cr` its per-cell rewards (or null), `tab` its table.
+template <int A, class Table, class ClassOf>
+__device__ __forceinline__ void run_env_steps(const Rules& R, const Ptrs& P, const int env,
+                                              const uint64_t t0, const int n_steps, ClassOf cls,
+                                              const float* __restrict__ cr, const Table tab) {
+  const int start = P.start[env];
+  const int sx = start % R.W, sy = start / R.W;
+  int s = P.s[env];
+  int x = s % R.W, y = s / R.W;
+  int ep_step = P.ep_step[env];
+  int episode = P.episode[env];
+  bool done = P.done[env] != 0;
+  float reward = 0.0f;
+  int action = 0;
+  Row<A> row = tab.load(s);
+  Philox4 blk = explore_block(R.seed, (uint32_t)env, t0 >> 1);
+
+  for (int k = 0; k < n_steps; ++k) {
+    const uint64_t t = t0 + (uint64_t)k;
+    Draw d = pick_draw(blk, t, A);
+    if (P.u_sup && t >= P.sup_t0 && t - P.sup_t0 < (uint64_t)P.sup_n) {
+      const size_t o = (size_t)(t - P.sup_t0) * P.N + env;
+      d.u = P.u_sup[o];
+      d.a = P.a_sup[o];
+    }
+    const float eps = eps_of(R, P.eps_tab, t, episode);
+    const int a = (d.u < eps) ? d.a : row_argmax(row);
+
+    const int s0 = s;
+    bool hit;
+    step_rule(R, cls, cr, x, y, a, reward, hit);
+    const int s2 = y * R.W + x;
+    done = hit || (!R.auto_reset && done);
+
+    // Q row of the new cell; when the env did not move it is the row in registers
+    Row<A> row2 = row;
+    if (s2 != s0) row2 = tab.load(s2);
+    // the next step's draws depend on nothing: the Philox rounds run while the
+    // row load is in flight
+    if ((t & 1) == 1) blk = explore_block(R.seed, (uint32_t)env, (t + 1) >> 1);
+    const float m = row_max(row2, done, R.max_mode);
+    const float qn = td_value(row_get(row, a), reward, m, R.lr, R.gamma);
+    tab.store(s0, a, qn);
+    if (s2 == s0) row2 = row_set(row2, a, qn);
+
+    ep_step += 1;
+    action = a;
+    if (env < P.trace_n && P.trace_cursor + k < P.trace_cap) {
+      const size_t o = (size_t)(P.trace_cursor + k) * P.trace_n + env;
+      P.tr_s[o] = s2;
+      P.tr_a[o] = (uint8_t)a;
+      P.tr_r[o] = reward;
+      P.tr_d[o] = done ? 1 : 0;
+    }
+    if (R.auto_reset && (done || (R.episode_len > 0 && ep_step >= R.episode_len))) {
+      x = sx;
+      y = sy;
+      s = start;
+      ep_step = 0;
+      episode += 1;
+      row = tab.load(start);
+      if (start == s0) row = row_set(row, a, qn);  // the value just written, from registers
+    } else {
+      s = s2;
+      row = row2;
+    }
+  }
+
+  P.s[env] = s;
+  P.ep_step[env] = ep_step;
+  P.episode[env] = episode;
+  P.reward[env] = reward;
+  P.done[env] = done ? 1 : 0;
+  P.action[env] = (uint8_t)action;
+}
+
+// The same loop for the common configuration, with everything that is fixed
+// there folded away: fixed epsilon, class rewards (no per-cell array), goal test
+// on the target cell, auto-reset, true max, no trace and no supplied stream.
+// Fewer live scalars and no optional branches: about half the instructions of
+// the general loop, which matters because a wave that waits for one row per
+// step is also issue-bound on the arithmetic between two rows.
+// `mapw(i)` returns word i of the env's packed map.
+template <int A, class Table, class MapWord>
+__device__ __forceinline__ void run_env_fast(const Rules& R, const Ptrs& P, const int env,
+                                             const uint64_t t0, const int n_steps, MapWord mapw,
+                                             const Table tab) {
+  const int W = R.W, H = R.H, T = R.episode_len;
+  const float eps = R.eps0, lr = R.lr, gamma = R.gamma;
+  const float r_step = R.step_reward, r_goal = R.goal_reward, r_trap = R.trap_reward;
+  const int start = P.start[env];
+  const int sx = start % W, sy = start / W;
+  int s = P.s[env];
+  int x = s % W, y = s / W;
+  int ep_step = P.ep_step[env];
+  int episode = P.episode[env];
+  float reward = 0.0f;
+  int action = 0;
+  bool hit = false;
+  Row<A> row = tab.load(s);
+  Philox4 blk = explore_block(R.seed, (uint32_t)env, t0 >> 1);
+  bool odd = (t0 & 1) != 0;
+  uint64_t next_block = (t0 >> 1) + 1;
+
+  for (int k = 0; k < n_steps; ++k) {
+    const uint32_t w0 = odd ? blk.w2 : blk.w0;
+    const uint32_t w1 = odd ? blk.w3 : blk.w1;
+    const int a = (u01(w0) < eps) ? (int)below(w1, (uint32_t)A) : row_argmax(row);
+
+    int dx, dy;
+    action_delta(a, A, dx, dy);
+    const int nx = x + dx, ny = y + dy;
+    const bool in = (unsigned)nx < (unsigned)W && (unsigned)ny < (unsigned)H;
+    const int tgt = in ? ny * W + nx : s;  // out of bounds: look at the own cell, result unused
+    const int cls = in ? cell_class_of(mapw(tgt >> 4), tgt) : kFree;
+    const bool moved = in && cls < kTrap;
+    x = moved ? nx : x;
+    y = moved ? ny : y;
+    const int s2 = moved ? tgt : s;
+    hit = cls == kGoal;
+    reward = hit ? r_goal : (cls == kTrap ? r_trap : r_step);
+
+    // the row of the cell the env stands on next; an env that stayed reads its own
+    // row again (still the pre-update values: the write below comes later)
+    Row<A> row2 = tab.load(s2);
+    if (odd) blk = explore_block(R.seed, (uint32_t)env, next_block++);  // in the load's shadow
+    const float m = row_max(row2, hit, 0);
+    const float qn = td_value(row_get(row, a), reward, m, lr, gamma);
+    tab.store(s, a, qn);
+    row2 = row_set(row2, s2 == s ? a : -1, qn);
+
+    action = a;
+    ep_step += 1;
+    odd = !odd;
+    if (hit || (T > 0 && ep_step >= T)) {
+      row = tab.load(start);
+      row = row_set(row, start == s ? a : -1, qn);  // the value just written, from registers
+      x = sx;
+      y = sy;
+      s = start;
+      ep_step = 0;
+      episode += 1;
+    } else {
+      s = s2;
+      row = row2;
+    }
+  }
+
+  P.s[env] = s;
+  P.ep_step[env] = ep_step;
+  P.episode[env] = episode;
+  P.reward[env] = reward;
+  P.done[env] = hit ? 1 : 0;
+  P.action[env] = (uint8_t)action;
+}
+
+// Per-env tables whose maps are shared (MAP = 1: the one map staged in LDS) or
+// too large for LDS (MAP = 2: read from global memory).  A block takes chunks
+// blockIdx, blockIdx + gridDim, ... and runs each for all n_steps.
 template <int A, int MAP>
 __global__ __launch_bounds__(256) void k_fused_per_env(const Rules R, const Ptrs P,
                                                         const uint64_t t0, const int n_steps) {
@@ -84,114 +254,123 @@ __global__ __launch_bounds__(256) void k_fused_per_env(const Rules R, const Ptrs
     for (int i = tid; i < P.map_words; i += bdim) lds[i] = P.map[i];
     __syncthreads();
   }
-
-  // A block takes chunks blockIdx, blockIdx + gridDim, ... and runs each for all
-  // n_steps.  The grid size therefore sets how many envs (and how many bytes of
-  // their tables) are live on the chip at once: small enough and the rows an
-  // env keeps returning to are still in the last-level cache.
   for (int chunk = blockIdx.x; chunk < n_chunks; chunk += gridDim.x) {
-    const int env0 = chunk * bdim;
-    const int env = env0 + tid;
-    const bool live = env < P.N;
-
-    if (MAP == 0) {
-      __syncthreads();  // the previous chunk's readers are done with the map
-      // the chunk's maps are contiguous in HBM: coalesced read, transposing write
-      const int n_here = min(bdim, P.N - env0);
-      const uint32_t* src = P.map + (size_t)env0 * P.map_words;
-      const int total = n_here * P.map_words;
-      for (int i = tid; i < total; i += bdim) {
-        const int e = i / P.map_words, w = i - e * P.map_words;
-        lds[w * bdim + e] = src[i];
-      }
-      __syncthreads();
-    }
-    if (!live) continue;  // only in the last chunk, after its barriers
-
+    const int env = chunk * bdim + tid;
+    if (env >= P.N) continue;
     const uint32_t* gmap = P.map + (P.map_shared ? 0 : (size_t)env * P.map_words);
     auto cls = [&](int cell) -> int {
-      uint32_t word;
-      if (MAP == 0)
-        word = lds[(cell >> 4) * bdim + tid];
-      else if (MAP == 1)
-        word = lds[cell >> 4];
-      else
-        word = gmap[cell >> 4];
+      const uint32_t word = (MAP == 1) ? lds[cell >> 4] : gmap[cell >> 4];
       return cell_class_of(word, cell);
     };
     const float* cr =
         P.cell_reward ? P.cell_reward + (P.map_shared ? 0 : (size_t)env * P.S) : nullptr;
+    run_env_steps<A>(R, P, env, t0, n_steps, cls, cr, GlobalTable<A>{P.Q + (size_t)env * P.S * A});
+  }
+}
 
-    float* __restrict__ Qe = P.Q + (size_t)env * P.S * A;
-    const int start = P.start[env];
-    const int sx = start % R.W, sy = start / R.W;
-    int s = P.s[env];
-    int x = s % R.W, y = s / R.W;
-    int ep_step = P.ep_step[env];
-    int episode = P.episode[env];
-    bool done = P.done[env] != 0;
-    float reward = 0.0f;
-    int action = 0;
-    Row<A> row = load_row<A>(Qe + (size_t)s * A);
-    Philox4 blk = explore_block(R.seed, (uint32_t)env, t0 >> 1);
+// Per-env tables with per-env maps small enough for LDS: every wave is an
+// independent worker that draws env ranges from one ticket counter (32 envs per
+// ticket), stages its envs' maps into its own LDS slice ([word][lane]: conflict
+// free) and steps them for all n_steps.  The grid size sets how many envs - and
+// how many bytes of their tables - are live on the chip at once: few enough and
+// the rows an env keeps returning to are still in the last-level cache.
+//
+// Waves 0-3 of a workgroup step 64 envs each against tables in HBM / the caches,
+// and spend most of their time waiting for one row per step.  With LDSW a fifth
+// wave uses the idle issue slots and the LDS: it stages the WHOLE tables of 32
+// envs into LDS, steps them there and writes the tables back.  The split between
+// the two kinds follows their speed; which worker steps an env does not change
+// its results.  FAST selects the folded loop (run_env_fast).
+constexpr int kTicketEnvs = 32;
 
-    for (int k = 0; k < n_steps; ++k) {
-      const uint64_t t = t0 + (uint64_t)k;
-      Draw d = pick_draw(blk, t, A);
-      if (P.u_sup && t >= P.sup_t0 && t - P.sup_t0 < (uint64_t)P.sup_n) {
-        const size_t o = (size_t)(t - P.sup_t0) * P.N + env;
-        d.u = P.u_sup[o];
-        d.a = P.a_sup[o];
+template <int A, bool FAST, bool LDSW>
+__global__ __launch_bounds__(LDSW ? 320 : 256) void k_fused_tickets(const Rules R, const Ptrs P,
+                                                                     const uint64_t t0,
+                                                                     const int n_steps,
+                                                                     unsigned* __restrict__ ticket,
+                                                                     const int tab_stride) {
+  extern __shared__ uint32_t lds[];
+  constexpr int kWaves = LDSW ? 5 : 4;
+  const int lane = threadIdx.x & 63;
+  const int wave = threadIdx.x >> 6;
+  uint32_t* my_map = lds + wave * (P.map_words * 64);  // [word][lane]
+  float* tabs = reinterpret_cast<float*>(lds + kWaves * (P.map_words * 64));
+  const unsigned n_tickets = (unsigned)((P.N + kTicketEnvs - 1) / kTicketEnvs);
+  const bool lds_worker = LDSW && wave == 4;
+  const int cap = lds_worker ? kTicketEnvs : 64;
+  const unsigned take = lds_worker ? 1u : 2u;
+  const size_t table = P.S * A;  // floats per table
+  auto mapw = [&](int word) -> uint32_t { return my_map[word * 64 + lane]; };
+  auto cls = [&](int cell) -> int { return cell_class_of(my_map[(cell >> 4) * 64 + lane], cell); };
+
+  while (true) {
+    unsigned base = 0;
+    if (lane == 0) base = atomicAdd(ticket, take);
+    base = __shfl(base, 0);
+    if (base >= n_tickets) break;  // every worker gets here: the counter only grows
+    const int env0 = (int)base * kTicketEnvs;
+    const int n_here = min(cap, P.N - env0);
+    const int env = env0 + lane;
+    const bool live = lane < n_here;
+    if (lane == 0) atomicAdd(ticket + (lds_worker ? 2 : 1), (unsigned)n_here);  // who did how much
+
+    // this worker's maps: contiguous in HBM, transposed into [word][lane]
+    __builtin_amdgcn_wave_barrier();
+    const uint32_t* src = P.map + (size_t)env0 * P.map_words;
+    for (int i = lane; i < n_here * P.map_words; i += 64) {
+      const int e = i / P.map_words, w = i - e * P.map_words;
+      my_map[w * 64 + e] = src[i];
+    }
+    const float* cr = P.cell_reward ? P.cell_reward + (size_t)env * P.S : nullptr;
+
+    if (!lds_worker) {
+      __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+      __builtin_amdgcn_wave_barrier();
+      if (live) {
+        const GlobalTable<A> tab{P.Q + (size_t)env * table};
+        if (FAST)
+          run_env_fast<A>(R, P, env, t0, n_steps, mapw, tab);
+        else
+          run_env_steps<A>(R, P, env, t0, n_steps, cls, cr, tab);
       }
-      const float eps = eps_of(R, P.eps_tab, t, episode);
-      const int a = (d.u < eps) ? d.a : row_argmax(row);
-
-      const int s0 = s;
-      bool hit;
-      step_rule(R, cls, cr, x, y, a, reward, hit);
-      const int s2 = y * R.W + x;
-      done = hit || (!R.auto_reset && done);
-
-      // Q row of the new cell; when the env did not move it is the row in registers
-      Row<A> row2 = row;
-      if (s2 != s0) row2 = load_row<A>(Qe + (size_t)s2 * A);
-      // the next step's draws depend on nothing: the Philox rounds run while the
-      // row load is in flight
-      if ((t & 1) == 1) blk = explore_block(R.seed, (uint32_t)env, (t + 1) >> 1);
-      const float m = row_max(row2, done, R.max_mode);
-      const float qn = td_value(row_get(row, a), reward, m, R.lr, R.gamma);
-      Qe[(size_t)s0 * A + a] = qn;
-      if (s2 == s0) row2 = row_set(row2, a, qn);
-
-      ep_step += 1;
-      action = a;
-      if (env < P.trace_n && P.trace_cursor + k < P.trace_cap) {
-        const size_t o = (size_t)(P.trace_cursor + k) * P.trace_n + env;
-        P.tr_s[o] = s2;
-        P.tr_a[o] = (uint8_t)a;
-        P.tr_r[o] = reward;
-        P.tr_d[o] = done ? 1 : 0;
+    } else {
+      // tables in: n_here consecutive tables are one contiguous run in HBM
+      const float4* g4 = reinterpret_cast<const float4*>(P.Q + (size_t)env0 * table);
+      const int t4 = (int)(table / 4);
+      const int total4 = n_here * t4;
+      for (int i0 = 0; i0 < total4; i0 += 64 * 8) {
+        float4 v[8];  // eight loads in flight per lane
+#pragma unroll
+        for (int u = 0; u < 8; ++u) {
+          const int i = i0 + u * 64 + lane;
+          if (i < total4) v[u] = g4[i];
+        }
+#pragma unroll
+        for (int u = 0; u < 8; ++u) {
+          const int i = i0 + u * 64 + lane;
+          if (i < total4) {
+            const int e = i / t4, o = i - e * t4;
+            reinterpret_cast<float4*>(tabs + e * tab_stride)[o] = v[u];
+          }
+        }
       }
-      if (R.auto_reset && (done || (R.episode_len > 0 && ep_step >= R.episode_len))) {
-        x = sx;
-        y = sy;
-        s = start;
-        ep_step = 0;
-        episode += 1;
-        row = load_row<A>(Qe + (size_t)start * A);
-        if (start == s0) row = row_set(row, a, qn);  // the value just written, from registers
-      } else {
-        s = s2;
-        row = row2;
+      __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+      __builtin_amdgcn_wave_barrier();
+      if (live) {
+        const LdsTable<A> tab{tabs + lane * tab_stride};
+        if (FAST)
+          run_env_fast<A>(R, P, env, t0, n_steps, mapw, tab);
+        else
+          run_env_steps<A>(R, P, env, t0, n_steps, cls, cr, tab);
+      }
+      __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+      __builtin_amdgcn_wave_barrier();
+      float4* o4 = reinterpret_cast<float4*>(P.Q + (size_t)env0 * table);
+      for (int i = lane; i < total4; i += 64) {
+        const int e = i / t4, o = i - e * t4;
+        o4[i] = reinterpret_cast<const float4*>(tabs + e * tab_stride)[o];
       }
     }
-
-    P.s[env] = s;
-    P.ep_step[env] = ep_step;
-    P.episode[env] = episode;
-    P.reward[env] = reward;
-    P.done[env] = done ? 1 : 0;
-    P.action[env] = (uint8_t)action;
   }
 }
 
@@ -424,6 +603,11 @@ __global__ __launch_bounds__(256) void k_shared_act(const Rules R, const Ptrs P,
     ReduceLds& L = *reinterpret_cast<ReduceLds*>(lds_raw);
     reduce_block(L, G, blockIdx.x, my_key, my_delta, live, handoff);
   }
+}
+
+__global__ void k_fill_u32(unsigned* p, const unsigned v, const int n) {
+  const int i = blockIdx.x * blockDim.x + threadIdx.x;
+  if (i < n) p[i] = v;
 }
 
 // plain copy of n16 16-byte words: the known-size launch that calibrates the

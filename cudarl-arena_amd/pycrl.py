@@ -78,7 +78,7 @@ _lib = None
 # every symbol include/crl.h declares
 EXPORTS = [
     "crl_last_error", "crl_version", "crl_device_count", "crl_create", "crl_destroy",
-    "crl_set_stream", "crl_sync", "crl_set_resident_envs", "crl_set_maps", "crl_set_cell", "crl_classify_grid", "crl_reset",
+    "crl_set_stream", "crl_sync", "crl_set_resident_envs", "crl_set_fused_variant", "crl_get_fused_split", "crl_set_maps", "crl_set_cell", "crl_classify_grid", "crl_reset",
     "crl_step", "crl_select", "crl_update", "crl_td_update", "crl_run_fused", "crl_get_state",
     "crl_set_state", "crl_get_step_count", "crl_set_step_count", "crl_q_get", "crl_q_set",
     "crl_q_get_range", "crl_set_trace", "crl_get_trace", "crl_set_exploration_stream",
@@ -104,6 +104,8 @@ def load():
     lib.crl_set_stream.argtypes = [vp, vp]
     lib.crl_sync.argtypes = [vp]
     lib.crl_set_resident_envs.argtypes = [vp, i32]
+    lib.crl_set_fused_variant.argtypes = [vp, i32]
+    lib.crl_get_fused_split.argtypes = [vp, C.POINTER(C.c_uint32), C.POINTER(C.c_uint32)]
     lib.crl_set_maps.argtypes = [vp, vp, vp, vp]
     lib.crl_set_cell.argtypes = [vp, i32, i32, i32, f32]
     lib.crl_classify_grid.argtypes = [vp, C.c_size_t, f32, vp, vp]
@@ -260,6 +262,14 @@ class Engine:
 
     def set_resident_envs(self, n):
         _check(self.lib.crl_set_resident_envs(self.h, n))
+
+    def set_fused_variant(self, v):
+        _check(self.lib.crl_set_fused_variant(self.h, v))
+
+    def fused_split(self):
+        a, b = C.c_uint32(), C.c_uint32()
+        _check(self.lib.crl_get_fused_split(self.h, C.byref(a), C.byref(b)))
+        return a.value, b.value
 
     def sync(self):
         _check(self.lib.crl_sync(self.h))

@@ -84,17 +84,20 @@ def test_fused_chunked_equals_one_launch(gpu, oracle):
 
 
 def test_fused_result_independent_of_resident_envs(gpu, oracle):
-    """Few envs in flight (blocks loop over chunks, re-staging maps) == all at once."""
-    N, W, H, T = 3000, 16, 16, 150
+    """Few envs in flight (blocks loop over chunks, re-staging maps) == all at once,
+    for the plain kernel and for the hybrid one (a fifth wave per workgroup steps
+    envs whose tables it holds in LDS; N is not a multiple of the 32-env ticket)."""
+    N, W, H, T = 3001, 16, 16, 150
     cls, start = gpu.gen_maps_bernoulli(31, N, N, W, H, 0.1, 0.02)
     cfg = gpu.make_config(N, W, H, episode_len=40, eps0=0.2, gamma=0.95, seed=17)
     outs = []
-    for resident in (0, 64, 640, 1000):
+    for resident, variant in ((0, 1), (64, 1), (640, 1), (1000, 1), (0, 2), (256, 2), (1024, 2)):
         with gpu.Engine(cfg, 0) as eng:
             eng.set_maps(cls, start)
             eng.set_resident_envs(resident)
-            if resident:
-                assert eng.fused_kernel_info()["grid"] == max(1, resident // eng.fused_kernel_info()["block"])
+            eng.set_fused_variant(variant)
+            info = eng.fused_kernel_info()
+            assert ("hbm+lds" in info["name"]) == (variant == 2), info
             eng.set_trace(N, T)
             eng.run_fused(T)
             outs.append((eng.get_trace(T), eng.q_get(0, N), eng.get_state()))
@@ -105,6 +108,39 @@ def test_fused_result_independent_of_resident_envs(gpu, oracle):
         assert_trace_equal(tr, want)
         assert_q_close(q, Q)
         assert np.array_equal(got["s"], st["s"]) and np.array_equal(got["episode"], st["episode"])
+
+
+@pytest.mark.parametrize("variant", [1, 2])
+@pytest.mark.parametrize("N,W,H,T,steps,t_odd", [(4097, 16, 16, 128, 300, 0), (700, 32, 32, 50, 401, 1),
+                                                 (33, 5, 7, 9, 77, 1)])
+def test_fused_fast_loop_matches_oracle(gpu, oracle, variant, N, W, H, T, steps, t_odd):
+    """Without a trace the common configuration runs the folded loop; final state
+    and tables must still be the oracle's, for waves on HBM tables and (variant 2)
+    the wave that steps envs from LDS-resident tables, from even and odd start steps."""
+    cls, start = gpu.gen_maps_bernoulli(41, N, N, W, H, 0.12, 0.03)
+    cfg = gpu.make_config(N, W, H, episode_len=T, eps0=0.15, gamma=0.95, seed=19, trap_reward=-1.0)
+    S = W * H
+    with gpu.Engine(cfg, 0) as eng:
+        eng.set_maps(cls, start)
+        eng.set_fused_variant(variant)
+        eng.step_count = t_odd
+        info = eng.fused_kernel_info()
+        assert "fast" in info["name"], info
+        if variant == 2 and S * 4 * 4 <= 4096:
+            assert "hbm+lds" in info["name"], info
+        eng.run_fused(steps // 2)
+        eng.run_fused(steps - steps // 2)
+        q, st = eng.q_get(0, N), eng.get_state()
+        hbm, lds = eng.fused_split()
+    if "hbm+lds" in info["name"] or True:
+        assert hbm + lds == N
+    Q = np.zeros((N, S, 4), np.float32)
+    ost = oracle.new_state(cfg, start)
+    oracle.run(cfg, cls, None, start, Q, ost, t_odd, steps)
+    for k in ("s", "ep_step", "episode", "reward", "done", "action"):
+        assert np.array_equal(st[k], ost[k]), k
+    assert_q_close(q.reshape(N, S, 4), Q)
+    assert st["episode"].max() >= 1
 
 
 def test_fused_large_map_global_path(gpu, oracle):
