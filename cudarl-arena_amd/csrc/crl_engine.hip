@@ -243,11 +243,22 @@ FusedPlan plan_fused(const crl_engine* e) {
     const size_t hybrid_lds = 5 * map_lds + (size_t)crl::kTicketEnvs * p.tab_stride * 4;
     const bool fits = e->K % 4 == 0 && hybrid_lds <= kLdsPerWorkgroup;
     p.hybrid = fits && (e->fused_variant == 2 || (e->fused_variant == 0 && e->N >= kHybridMinEnvs));
-    p.block = p.hybrid ? 320 : 256;
-    p.lds = p.hybrid ? hybrid_lds : 4 * map_lds;
     const long tickets = (e->N + crl::kTicketEnvs - 1) / crl::kTicketEnvs;
-    const long per_wg = p.hybrid ? 9 : 8;  // tickets one workgroup takes per round
-    p.grid = (int)std::min<long>(std::max<long>(1, resident / 256), (tickets + per_wg - 1) / per_wg);
+    if (p.hybrid) {
+      p.block = 320;
+      p.lds = hybrid_lds;
+      p.grid = (int)std::min<long>(std::max<long>(1, resident / 256), (tickets + 8) / 9);
+    } else if (tickets / 2 < 4 * 256) {
+      // fewer 64-env workers than SIMDs on the chip: one-wave workgroups spread
+      // them over the compute units instead of packing four per unit
+      p.block = 64;
+      p.lds = map_lds;
+      p.grid = (int)std::min<long>(std::max<long>(1, resident / 64), (tickets + 1) / 2);
+    } else {
+      p.block = 256;
+      p.lds = 4 * map_lds;
+      p.grid = (int)std::min<long>(std::max<long>(1, resident / 256), (tickets + 7) / 8);
+    }
   }
   static const char* names[2][3] = {
       {"k_fused_per_env<4,0>", "k_fused_per_env<4,1>", "k_fused_per_env<4,2>"},
