@@ -190,14 +190,17 @@ __device__ __forceinline__ void run_env_fast(const Rules& R, const Ptrs& P, cons
   for (int k = 0; k < n_steps; ++k) {
     const uint32_t w0 = odd ? blk.w2 : blk.w0;
     const uint32_t w1 = odd ? blk.w3 : blk.w1;
-    const int a = (u01(w0) < eps) ? (int)below(w1, (uint32_t)A) : row_argmax(row);
+    // both candidates are computed and one is selected: cheaper than a divergent branch
+    const int greedy = row_argmax(row);
+    const int a = (u01(w0) < eps) ? (int)below(w1, (uint32_t)A) : greedy;
 
     int dx, dy;
     action_delta(a, A, dx, dy);
     const int nx = x + dx, ny = y + dy;
     const bool in = (unsigned)nx < (unsigned)W && (unsigned)ny < (unsigned)H;
     const int tgt = in ? ny * W + nx : s;  // out of bounds: look at the own cell, result unused
-    const int cls = in ? cell_class_of(mapw(tgt >> 4), tgt) : kFree;
+    const int looked = cell_class_of(mapw(tgt >> 4), tgt);
+    const int cls = in ? looked : kFree;
     const bool moved = in && cls < kTrap;
     x = moved ? nx : x;
     y = moved ? ny : y;
