@@ -229,3 +229,84 @@ def test_engine_argument_errors(gpu):
         assert eng.step_count == 0
     with pytest.raises(gpu.CrlError):
         gpu.Engine(cfg, 99)
+
+
+# ---- the batched pybind surface (additive: cudarl_core.BatchedEnvironment) ----------
+
+def test_batched_environment_matches_oracle(core, gpu, oracle):
+    N, W, H, T = 500, 12, 12, 120
+    cls, start = gpu.gen_maps_bernoulli(3, N, N, W, H, 0.15, 0.03)
+    env = core.BatchedEnvironment(N, W, H, learning_rate=0.1, discount_factor=0.95, exploration_rate=0.2,
+                                  episode_len=30, seed=5)
+    assert (env.num_envs, env.num_states, env.num_actions, env.num_tables) == (N, W * H, 4, N)
+    env.set_maps(cls, start)
+    env.run(T // 2)
+    for _ in range(T - T // 2):  # the rest through the decomposed calls
+        a = env.select()
+        assert a.dtype == np.int32 and a.shape == (N,)
+        env.step()
+        env.update()
+    assert env.step_count == T
+    cfg = gpu.make_config(N, W, H, lr=0.1, gamma=0.95, eps0=0.2, episode_len=30, seed=5)
+    Q = np.zeros((N, W * H, 4), np.float32)
+    st = oracle.new_state(cfg, start)
+    oracle.run(cfg, cls, None, start, Q, st, 0, T)
+    got = env.state()
+    for k in ("s", "ep_step", "episode", "reward", "done", "action"):
+        assert np.array_equal(got[k], st[k]), k
+    for t in (0, 7, N - 1):
+        q = env.q_table(t)
+        assert q.shape == (W * H, 4) and np.array_equal(q, Q[t])
+    env.set_q_table(3, np.ones((W * H, 4), np.float32))
+    assert (env.q_table(3) == 1).all()
+    with pytest.raises(RuntimeError):
+        env.set_maps(cls[:10], start)
+    with pytest.raises(RuntimeError):
+        env.step(np.zeros(3, np.int32))
+
+
+def test_batched_environment_dlpack_views(core, gpu):
+    """Zero-copy views: a DLPack capsule per SoA array that points at the engine's
+    own device memory (ROCm device type 10), checked field by field and by copying
+    the bytes back with hipMemcpy."""
+    import ctypes as C
+    N, W, H = 300, 8, 8
+    cls, start = gpu.gen_maps_bernoulli(1, N, N, W, H, 0.1)
+    env = core.BatchedEnvironment(N, W, H, exploration_rate=0.3, episode_len=20, seed=2)
+    env.set_maps(cls, start)
+    env.run(50)
+    env.sync()
+    st = env.state()
+
+    class DLTensor(C.Structure):
+        _fields_ = [("data", C.c_void_p), ("device_type", C.c_int32), ("device_id", C.c_int32),
+                    ("ndim", C.c_int32), ("code", C.c_uint8), ("bits", C.c_uint8), ("lanes", C.c_uint16),
+                    ("shape", C.POINTER(C.c_int64)), ("strides", C.POINTER(C.c_int64)),
+                    ("byte_offset", C.c_uint64)]
+
+    get = C.pythonapi.PyCapsule_GetPointer
+    get.restype, get.argtypes = C.c_void_p, [C.py_object, C.c_char_p]
+    hip = C.CDLL("libamdhip64.so")
+    hip.hipMemcpy.argtypes = [C.c_void_p, C.c_void_p, C.c_size_t, C.c_int]
+    for name, dtype, code, bits in (("s", np.int32, 0, 32), ("reward", np.float32, 2, 32),
+                                    ("done", np.uint8, 1, 8), ("action", np.uint8, 1, 8),
+                                    ("episode", np.int32, 0, 32)):
+        cap = env.dlpack(name)
+        t = DLTensor.from_address(get(cap, b"dltensor"))
+        assert (t.device_type, t.device_id, t.ndim, t.code, t.bits, t.lanes) == (10, 0, 1, code, bits, 1)
+        assert t.shape[0] == N and not t.strides and t.byte_offset == 0
+        assert t.data == env.device_pointer(name)
+        host = np.empty(N, dtype)
+        assert hip.hipMemcpy(host.ctypes.data, t.data, host.nbytes, 2) == 0
+        assert np.array_equal(host, st[name]), name
+        del cap  # an unconsumed capsule frees its tensor
+    cap = env.dlpack("q")
+    t = DLTensor.from_address(get(cap, b"dltensor"))
+    assert (t.ndim, t.shape[0], t.shape[1], t.shape[2]) == (3, N, W * H, 4)
+    host = np.empty((W * H, 4), np.float32)
+    assert hip.hipMemcpy(host.ctypes.data, t.data + 5 * host.nbytes, host.nbytes, 2) == 0
+    assert np.array_equal(host, env.q_table(5))
+    del env  # the view keeps the engine alive
+    assert hip.hipMemcpy(host.ctypes.data, t.data, host.nbytes, 2) == 0
+    with pytest.raises(RuntimeError):
+        core.BatchedEnvironment(4, 4, 4).dlpack("nope")
