@@ -7,7 +7,7 @@ One "step" advances every env of the workload by one select -> step -> update.
 W warm-up steps run first, then exactly K steps are timed with the inputs (maps,
 tables, state) already resident in HBM.  Prints ONE JSON line.
 
-Workloads (BASELINE.json configs, 1-based as in BASELINE.md):
+Workloads (the benchmark configurations, numbered from 1):
   c2  4096 envs, 32x32, per-env tables (64 MB; cache resident)
   c3  65536 envs sharing one 64x64 map and ONE table (ordered reduction per step)
   c4  1,048,576 envs, 16x16, per-env tables (4 GB; the HBM-bound config)  [default]

@@ -20,6 +20,7 @@ struct Rules {
   int max_mode;  // 0 true max, 1 zero floor
   int eps_mode;  // 0 fixed, 1 by global step, 2/3 by per-env episode
   int eps_len;
+  int max_episodes;  // > 0: envs that finished this many episodes stop stepping
   float lr, gamma;
   float step_reward, goal_reward, trap_reward;
   float eps0;

@@ -85,6 +85,9 @@ struct crl_engine {
   DevBuf<float> Q;
   DevBuf<float> eps_tab;
   int eps_len = 1;
+  // episode statistics (allocated when cfg.track_returns)
+  DevBuf<float> ret_acc, ret_last, ret_sum;
+  DevBuf<int32_t> len_last, len_sum;
   // transition of the last crl_step
   DevBuf<int32_t> tr_s, tr_a, tr_s2;
   DevBuf<float> tr_r;
@@ -126,6 +129,7 @@ struct crl_engine {
     R.max_mode = cfg.max_mode;
     R.eps_mode = cfg.eps_mode;
     R.eps_len = eps_len;
+    R.max_episodes = cfg.max_episodes;
     R.lr = cfg.lr;
     R.gamma = cfg.gamma;
     R.step_reward = cfg.step_reward;
@@ -159,6 +163,11 @@ struct crl_engine {
     P.trace_n = trace_n;
     P.trace_cursor = trace_cursor;
     P.trace_cap = trace_cap;
+    P.ret_acc = ret_acc.p;
+    P.ret_last = ret_last.p;
+    P.ret_sum = ret_sum.p;
+    P.len_last = len_last.p;
+    P.len_sum = len_sum.p;
     P.N = N;
     P.map_words = map_words;
     P.map_shared = cfg.map_mode == CRL_MAP_SHARED;
@@ -235,7 +244,8 @@ FusedPlan plan_fused(const crl_engine* e) {
   } else {
     const crl_config& c = e->cfg;
     p.fast = c.eps_mode == CRL_EPS_FIXED && c.reward_flags == 0 && c.goal_mode == CRL_GOAL_ON_TARGET &&
-             c.auto_reset == 1 && c.max_mode == CRL_MAX_TRUE && e->trace_n == 0 && e->sup_n == 0;
+             c.auto_reset == 1 && c.max_mode == CRL_MAX_TRUE && e->trace_n == 0 && e->sup_n == 0 &&
+             c.max_episodes == 0 && c.track_returns == 0;
     // Hybrid workgroups when 32 whole tables (padded by one row against bank
     // conflicts) and five waves' maps fit into LDS.
     p.tab_stride = (int)e->K + 4;
@@ -526,6 +536,13 @@ int crl_create(const crl_config* cfg, int device, crl_engine** out) {
     acc(e->key.alloc(N));
     acc(e->delta.alloc(N));
   }
+  if (cfg->track_returns) {
+    acc(e->ret_acc.alloc(N));
+    acc(e->ret_last.alloc(N));
+    acc(e->ret_sum.alloc(N));
+    acc(e->len_last.alloc(N));
+    acc(e->len_sum.alloc(N));
+  }
   if (a != hipSuccess) {
     const int code = a == hipErrorOutOfMemory ? CRL_E_ALLOC : CRL_E_DEVICE;
     delete e;
@@ -554,6 +571,11 @@ int crl_create(const crl_config* cfg, int device, crl_engine** out) {
   if ((h = hipMemsetAsync(e->done.p, 0, N, e->stream)) != hipSuccess) return bail(h, "clear");
   if ((h = hipMemsetAsync(e->action.p, 0, N, e->stream)) != hipSuccess) return bail(h, "clear");
   if ((h = hipMemsetAsync(e->map.p, 0, e->map.n * 4, e->stream)) != hipSuccess) return bail(h, "clear");
+  if (cfg->track_returns) {
+    void* bufs[] = {e->ret_acc.p, e->ret_last.p, e->ret_sum.p, e->len_last.p, e->len_sum.p};
+    for (void* b : bufs)
+      if ((h = hipMemsetAsync(b, 0, N * 4, e->stream)) != hipSuccess) return bail(h, "clear");
+  }
   if ((h = hipMemcpyAsync(e->eps_tab.p, eps.data(), eps.size() * sizeof(float), hipMemcpyHostToDevice,
                           e->stream)) != hipSuccess)
     return bail(h, "upload eps table");
@@ -866,6 +888,20 @@ int crl_set_state(crl_engine* e, const int32_t* s, const int32_t* ep_step, const
   HIP_TRY(hipStreamSynchronize(e->stream));
   e->have_transition = false;
   e->have_actions = false;
+  return CRL_OK;
+}
+
+int crl_get_episode_stats(crl_engine* e, float* last_return, int32_t* last_length, float* return_sum,
+                          int32_t* length_sum) {
+  int rc = check_engine(e);
+  if (rc) return rc;
+  if (!e->cfg.track_returns) return fail(CRL_E_STATE, "the engine was created without track_returns");
+  const size_t b = (size_t)e->N * 4;
+  if (last_return) HIP_TRY(hipMemcpyAsync(last_return, e->ret_last.p, b, hipMemcpyDeviceToHost, e->stream));
+  if (last_length) HIP_TRY(hipMemcpyAsync(last_length, e->len_last.p, b, hipMemcpyDeviceToHost, e->stream));
+  if (return_sum) HIP_TRY(hipMemcpyAsync(return_sum, e->ret_sum.p, b, hipMemcpyDeviceToHost, e->stream));
+  if (length_sum) HIP_TRY(hipMemcpyAsync(length_sum, e->len_sum.p, b, hipMemcpyDeviceToHost, e->stream));
+  HIP_TRY(hipStreamSynchronize(e->stream));
   return CRL_OK;
 }
 

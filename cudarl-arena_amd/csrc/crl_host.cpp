@@ -43,6 +43,8 @@ int validate_config(const crl_config* c, std::string& why) {
   if (c->eps_mode < CRL_EPS_FIXED || c->eps_mode > CRL_EPS_EPISODE_LINEAR) return bad(CRL_E_ARG, "bad eps_mode");
   if (c->eps_mode != CRL_EPS_FIXED && c->eps_span < 1) return bad(CRL_E_ARG, "eps_span must be >= 1");
   if (c->eps_span > (1 << 26)) return bad(CRL_E_ARG, "eps_span too large");
+  if (c->max_episodes < 0) return bad(CRL_E_ARG, "max_episodes must be >= 0");
+  if (c->track_returns != 0 && c->track_returns != 1) return bad(CRL_E_ARG, "track_returns must be 0 or 1");
   if ((uint64_t)c->n_envs * (uint64_t)c->width * c->height > ((uint64_t)1 << 40))
     return bad(CRL_E_ARG, "n_envs * cells too large");
   return CRL_OK;

@@ -38,6 +38,13 @@ struct Ptrs {
   float* tr_r;
   uint8_t* tr_d;
   int trace_n, trace_cursor, trace_cap;
+  // episode statistics (all null unless tracked): running return of the open
+  // episode, return / length of the last finished one, sums over finished ones
+  float* ret_acc;
+  float* ret_last;
+  float* ret_sum;
+  int32_t* len_last;
+  int32_t* len_sum;
   // geometry
   int N;
   int map_words;   // uint32 words per map
@@ -45,6 +52,25 @@ struct Ptrs {
   int table_shared;  // 1: one table for all envs
   size_t S;        // cells per map
 };
+
+// an episode of `env` just ended with return `ret` after `len` steps
+__device__ __forceinline__ void record_episode(const Ptrs& P, int env, float ret, int len) {
+  P.ret_last[env] = ret;
+  P.len_last[env] = len;
+  P.ret_sum[env] = P.ret_sum[env] + ret;
+  P.len_sum[env] = P.len_sum[env] + len;
+}
+
+// trace row of an env that has used up its episode budget: it stays where it is
+__device__ __forceinline__ void trace_idle(const Ptrs& P, int env, int row, int s) {
+  if (env < P.trace_n && row < P.trace_cap) {
+    const size_t o = (size_t)row * P.trace_n + env;
+    P.tr_s[o] = s;
+    P.tr_a[o] = 0;
+    P.tr_r[o] = 0.0f;
+    P.tr_d[o] = 0;
+  }
+}
 
 // the two draws of step t for one env
 struct Draw {
@@ -95,12 +121,19 @@ __device__ __forceinline__ void run_env_steps(const Rules& R, const Ptrs& P, con
   int ep_step = P.ep_step[env];
   int episode = P.episode[env];
   bool done = P.done[env] != 0;
-  float reward = 0.0f;
-  int action = 0;
+  float reward = P.reward[env];  // rewritten unchanged if the env's episode budget is used up
+  int action = P.action[env];
   Row<A> row = tab.load(s);
   Philox4 blk = explore_block(R.seed, (uint32_t)env, t0 >> 1);
+  const bool track = P.ret_acc != nullptr;
+  float ret = track ? P.ret_acc[env] : 0.0f;
 
   for (int k = 0; k < n_steps; ++k) {
+    if (R.max_episodes > 0 && episode >= R.max_episodes) {
+      // budget used up: for ever, so the rest of the launch only fills the trace
+      for (int kk = k; kk < n_steps; ++kk) trace_idle(P, env, P.trace_cursor + kk, s);
+      break;
+    }
     const uint64_t t = t0 + (uint64_t)k;
     Draw d = pick_draw(blk, t, A);
     if (P.u_sup && t >= P.sup_t0 && t - P.sup_t0 < (uint64_t)P.sup_n) {
@@ -130,6 +163,7 @@ __device__ __forceinline__ void run_env_steps(const Rules& R, const Ptrs& P, con
 
     ep_step += 1;
     action = a;
+    ret = ret + reward;
     if (env < P.trace_n && P.trace_cursor + k < P.trace_cap) {
       const size_t o = (size_t)(P.trace_cursor + k) * P.trace_n + env;
       P.tr_s[o] = s2;
@@ -138,6 +172,8 @@ __device__ __forceinline__ void run_env_steps(const Rules& R, const Ptrs& P, con
       P.tr_d[o] = done ? 1 : 0;
     }
     if (R.auto_reset && (done || (R.episode_len > 0 && ep_step >= R.episode_len))) {
+      if (track) record_episode(P, env, ret, ep_step);
+      ret = 0.0f;
       x = sx;
       y = sy;
       s = start;
@@ -154,6 +190,7 @@ __device__ __forceinline__ void run_env_steps(const Rules& R, const Ptrs& P, con
   P.s[env] = s;
   P.ep_step[env] = ep_step;
   P.episode[env] = episode;
+  if (track) P.ret_acc[env] = ret;
   P.reward[env] = reward;
   P.done[env] = done ? 1 : 0;
   P.action[env] = (uint8_t)action;
@@ -436,6 +473,15 @@ __global__ __launch_bounds__(256) void k_step(const Rules R, const Ptrs P, const
   auto cls = [&](int cell) -> int { return cell_class_of(gmap[cell >> 4], cell); };
   const float* cr = P.cell_reward ? P.cell_reward + (P.map_shared ? 0 : (size_t)env * P.S) : nullptr;
   const int s0 = P.s[env];
+  if (R.max_episodes > 0 && P.episode[env] >= R.max_episodes) {
+    T.s[env] = s0;  // budget used up: no move and, with action -1, no update
+    T.a[env] = -1;
+    T.r[env] = 0.0f;
+    T.s2[env] = s0;
+    T.done[env] = 0;
+    trace_idle(P, env, P.trace_cursor, s0);
+    return;
+  }
   int x = s0 % R.W, y = s0 / R.W;
   const int a = act[env];
   float reward;
@@ -444,6 +490,7 @@ __global__ __launch_bounds__(256) void k_step(const Rules R, const Ptrs P, const
   const int s2 = y * R.W + x;
   const bool done = hit || (!R.auto_reset && P.done[env] != 0);
   int ep_step = P.ep_step[env] + 1;
+  const float ret = P.ret_acc ? P.ret_acc[env] + reward : 0.0f;
   T.s[env] = s0;
   T.a[env] = a;
   T.r[env] = reward;
@@ -460,10 +507,15 @@ __global__ __launch_bounds__(256) void k_step(const Rules R, const Ptrs P, const
     P.tr_d[o] = done ? 1 : 0;
   }
   if (R.auto_reset && (done || (R.episode_len > 0 && ep_step >= R.episode_len))) {
+    if (P.ret_acc) {
+      record_episode(P, env, ret, ep_step);
+      P.ret_acc[env] = 0.0f;
+    }
     P.s[env] = P.start[env];
     P.ep_step[env] = 0;
     P.episode[env] += 1;
   } else {
+    if (P.ret_acc) P.ret_acc[env] = ret;
     P.s[env] = s2;
     P.ep_step[env] = ep_step;
   }
@@ -479,6 +531,7 @@ __global__ __launch_bounds__(256) void k_reset(const Ptrs P, const int first, co
   P.reward[env] = 0.0f;
   P.done[env] = 0;
   P.action[env] = 0;
+  if (P.ret_acc) P.ret_acc[env] = 0.0f;
 }
 
 // TD update of one recorded transition per env on the env's own table
@@ -539,7 +592,7 @@ __global__ __launch_bounds__(256) void k_shared_act(const Rules R, const Ptrs P,
   uint32_t* lds_map = reinterpret_cast<uint32_t*>(lds_raw + (REDUCE ? sizeof(ReduceLds) : 0));
   const int tid = threadIdx.x;
   const int env = blockIdx.x * blockDim.x + tid;
-  const bool live = env < P.N;
+  bool live = env < P.N;
   // the env's cell is fetched while the map streams into LDS
   const int s_in = live ? P.s[env] : 0;
   if (MAP == 1) {
@@ -548,6 +601,12 @@ __global__ __launch_bounds__(256) void k_shared_act(const Rules R, const Ptrs P,
   }
   int my_key = 0;
   float my_delta = 0.0f;
+  if (live && R.max_episodes > 0 && P.episode[env] >= R.max_episodes) {
+    live = false;  // budget used up: no move, no delta
+    key[env] = -1;
+    delta[env] = 0.0f;
+    trace_idle(P, env, trace_row, s_in);
+  }
   if (live) {
     const uint32_t* gmap = P.map + (P.map_shared ? 0 : (size_t)env * P.map_words);
     auto cls = [&](int cell) -> int {
@@ -593,11 +652,17 @@ __global__ __launch_bounds__(256) void k_shared_act(const Rules R, const Ptrs P,
       P.tr_r[o] = reward;
       P.tr_d[o] = done ? 1 : 0;
     }
+    const float ret = P.ret_acc ? P.ret_acc[env] + reward : 0.0f;
     if (R.auto_reset && (done || (R.episode_len > 0 && ep_step >= R.episode_len))) {
+      if (P.ret_acc) {
+        record_episode(P, env, ret, ep_step);
+        P.ret_acc[env] = 0.0f;
+      }
       P.s[env] = P.start[env];
       P.ep_step[env] = 0;
       P.episode[env] = episode + 1;
     } else {
+      if (P.ret_acc) P.ret_acc[env] = ret;
       P.s[env] = s2;
       P.ep_step[env] = ep_step;
     }

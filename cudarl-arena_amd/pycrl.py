@@ -46,6 +46,8 @@ class Config(C.Structure):
         ("eps_decay", C.c_float),
         ("eps_end", C.c_float),
         ("eps_span", C.c_int32),
+        ("max_episodes", C.c_int32),
+        ("track_returns", C.c_int32),
         ("seed", C.c_uint64),
     ]
 
@@ -53,7 +55,8 @@ class Config(C.Structure):
 def make_config(n_envs, width, height, n_actions=4, table_mode=TABLE_PER_ENV, map_mode=MAP_PER_ENV,
                 max_mode=MAX_TRUE, goal_mode=GOAL_ON_TARGET, auto_reset=1, episode_len=0, lr=0.1,
                 gamma=0.99, step_reward=-0.01, goal_reward=1.0, trap_reward=-1.0, reward_flags=0,
-                eps_mode=EPS_FIXED, eps0=0.1, eps_decay=1.0, eps_end=0.0, eps_span=1, seed=0):
+                eps_mode=EPS_FIXED, eps0=0.1, eps_decay=1.0, eps_end=0.0, eps_span=1, seed=0,
+                max_episodes=0, track_returns=0):
     c = Config()
     c.struct_size = C.sizeof(Config)
     c.n_envs, c.width, c.height, c.n_actions = n_envs, width, height, n_actions
@@ -63,6 +66,7 @@ def make_config(n_envs, width, height, n_actions=4, table_mode=TABLE_PER_ENV, ma
     c.step_reward, c.goal_reward, c.trap_reward = step_reward, goal_reward, trap_reward
     c.reward_flags, c.eps_mode = reward_flags, eps_mode
     c.eps0, c.eps_decay, c.eps_end, c.eps_span = eps0, eps_decay, eps_end, eps_span
+    c.max_episodes, c.track_returns = max_episodes, track_returns
     c.seed = seed
     return c
 
@@ -80,7 +84,7 @@ EXPORTS = [
     "crl_last_error", "crl_version", "crl_device_count", "crl_create", "crl_destroy",
     "crl_set_stream", "crl_sync", "crl_set_resident_envs", "crl_set_fused_variant", "crl_get_fused_split", "crl_set_maps", "crl_set_cell", "crl_classify_grid", "crl_reset",
     "crl_step", "crl_select", "crl_update", "crl_td_update", "crl_run_fused", "crl_get_state",
-    "crl_set_state", "crl_get_step_count", "crl_set_step_count", "crl_q_get", "crl_q_set",
+    "crl_set_state", "crl_get_episode_stats", "crl_get_step_count", "crl_set_step_count", "crl_q_get", "crl_q_set",
     "crl_q_get_range", "crl_set_trace", "crl_get_trace", "crl_set_exploration_stream",
     "crl_device_ptr", "crl_fused_kernel_info", "crl_philox4x32_10", "crl_explore_draw",
     "crl_eps_table", "crl_gen_maps_bernoulli", "crl_gen_maps_noise", "crl_probe_copy",
@@ -117,6 +121,7 @@ def load():
     lib.crl_run_fused.argtypes = [vp, i32]
     lib.crl_get_state.argtypes = [vp, vp, vp, vp, vp, vp, vp]
     lib.crl_set_state.argtypes = [vp, vp, vp, vp]
+    lib.crl_get_episode_stats.argtypes = [vp, vp, vp, vp, vp]
     lib.crl_get_step_count.argtypes = [vp, C.POINTER(u64)]
     lib.crl_set_step_count.argtypes = [vp, u64]
     lib.crl_q_get.argtypes = [vp, i32, vp]
@@ -281,6 +286,14 @@ class Engine:
                    episode=np.empty(N, np.int32))
         _check(self.lib.crl_get_state(self.h, _ptr(out["s"]), _ptr(out["reward"]), _ptr(out["done"]),
                                       _ptr(out["action"]), _ptr(out["ep_step"]), _ptr(out["episode"])))
+        return out
+
+    def episode_stats(self):
+        N = self.N
+        out = dict(last_return=np.empty(N, np.float32), last_length=np.empty(N, np.int32),
+                   return_sum=np.empty(N, np.float32), length_sum=np.empty(N, np.int32))
+        _check(self.lib.crl_get_episode_stats(self.h, _ptr(out["last_return"]), _ptr(out["last_length"]),
+                                              _ptr(out["return_sum"]), _ptr(out["length_sum"])))
         return out
 
     def set_state(self, s=None, ep_step=None, episode=None):

@@ -92,6 +92,11 @@ typedef struct crl_config {
   int32_t eps_mode;      /* CRL_EPS_*                                              */
   float eps0, eps_decay, eps_end;
   int32_t eps_span;      /* table length for the STEP/EPISODE schedules            */
+  int32_t max_episodes;  /* > 0: an env stops stepping once it has finished this
+                            many episodes (the `for episode in range(num_episodes)`
+                            of src/train.py:191); 0 = no budget                    */
+  int32_t track_returns; /* 1: keep per-env episode return / length accumulators
+                            on the device (src/train.py:205-226)                   */
   uint64_t seed;         /* Philox4x32-10 key                                      */
 } crl_config;
 
@@ -191,6 +196,13 @@ int crl_get_state(crl_engine* e, int32_t* s, float* reward, uint8_t* done, uint8
  * get/set_q_table).  Any pointer may be NULL. */
 int crl_set_state(crl_engine* e, const int32_t* s, const int32_t* ep_step,
                   const int32_t* episode);
+/* Episode statistics (needs track_returns): return and length of the last
+ * finished episode of every env, and their sums over all finished episodes
+ * (the number of finished episodes is `episode` of crl_get_state).  Any pointer
+ * may be NULL.  Replaces the episode_rewards / episode_lengths lists of
+ * src/train.py:186-226. */
+int crl_get_episode_stats(crl_engine* e, float* last_return, int32_t* last_length,
+                          float* return_sum, int32_t* length_sum);
 /* global step counter t (number of updates so far) */
 int crl_get_step_count(crl_engine* e, uint64_t* t);
 int crl_set_step_count(crl_engine* e, uint64_t t);

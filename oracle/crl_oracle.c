@@ -52,6 +52,8 @@ typedef struct orc_config {
   int32_t eps_mode;     /* 0 fixed, 1 step mult, 2 episode mult, 3 episode linear */
   float eps0, eps_decay, eps_end;
   int32_t eps_span;
+  int32_t max_episodes;  /* > 0: an env stops after this many episodes (src/train.py:191) */
+  int32_t track_returns; /* informational here: the stats arrays are passed explicitly */
   uint64_t seed;
 } orc_config;
 
@@ -456,14 +458,30 @@ static int eps_cap(const orc_config* c) {
   return 1;
 }
 
+/* per-env episode statistics (src/train.py:186-226: episode_reward summed step
+ * by step, episode_rewards / episode_lengths appended when the episode ends);
+ * every pointer indexes one env, or the struct pointer is NULL */
+typedef struct {
+  float* ret_acc;    /* return of the open episode */
+  float* ret_last;   /* return of the last finished episode */
+  float* ret_sum;    /* sum over finished episodes */
+  int32_t* len_last;
+  int32_t* len_sum;
+} orc_stats;
+
 /* One env, one step: select (src/train.py:200) -> step (:201) -> update (:205).
  * q is the env's table (or the shared one); with sum != NULL the delta goes
- * into the ordered tree instead of being applied.  Returns s' before any restart. */
+ * into the ordered tree instead of being applied.  Returns s' before any
+ * restart, or -1 if the env has used up its episode budget and did nothing. */
 static int32_t env_step(const orc_config* c, float eps, float u, int32_t ar, const uint8_t* m_cls,
                         const float* m_cr, float* q, orc_tree* sum, int32_t start, int32_t* s,
                         int32_t* ep_step, int32_t* episode, float* reward, uint8_t* done,
-                        uint8_t* action) {
+                        uint8_t* action, const orc_stats* st) {
   const int A = c->n_actions;
+  if (c->max_episodes > 0 && *episode >= c->max_episodes) {
+    if (sum) tree_add(sum, -1, 0.0f);
+    return -1;
+  }
   int32_t s0 = *s;
   int a = orc_select(q + (size_t)s0 * A, A, eps, u, ar);
   int32_t s2 = s0;
@@ -480,7 +498,15 @@ static int32_t env_step(const orc_config* c, float eps, float u, int32_t ar, con
   *reward = r;
   *done = (uint8_t)d;
   *action = (uint8_t)a;
+  if (st) *st->ret_acc = *st->ret_acc + r;
   if (c->auto_reset && (d || (c->episode_len > 0 && *ep_step >= c->episode_len))) {
+    if (st) {
+      *st->ret_last = *st->ret_acc;
+      *st->len_last = *ep_step;
+      *st->ret_sum = *st->ret_sum + *st->ret_acc;
+      *st->len_sum = *st->len_sum + *ep_step;
+      *st->ret_acc = 0.0f;
+    }
     *s = start;
     *ep_step = 0;
     *episode += 1;
@@ -505,7 +531,8 @@ int orc_run(const orc_config* c, const uint8_t* cls, const float* cr, const int3
             float* Q, int32_t* s, int32_t* ep_step, int32_t* episode, float* reward,
             uint8_t* done, uint8_t* action, uint64_t t0, int32_t n_steps, const float* u_sup,
             const int32_t* a_sup, int32_t trace_n, int32_t* tr_s, uint8_t* tr_a, float* tr_r,
-            uint8_t* tr_d) {
+            uint8_t* tr_d, float* ret_acc, float* ret_last, float* ret_sum, int32_t* len_last,
+            int32_t* len_sum) {
   const int N = c->n_envs, A = c->n_actions;
   const size_t S = (size_t)c->width * c->height;
   const size_t K = S * A;
@@ -535,15 +562,30 @@ int orc_run(const orc_config* c, const uint8_t* cls, const float* cr, const int3
         orc_explore_draw(c->seed, (uint32_t)i, t, A, &u, &ar);
       }
       float eps = eps_at(c, tab, len, t, episode[i]);
+      orc_stats st = {0};
+      if (ret_acc) {
+        st.ret_acc = ret_acc + i;
+        st.ret_last = ret_last + i;
+        st.ret_sum = ret_sum + i;
+        st.len_last = len_last + i;
+        st.len_sum = len_sum + i;
+      }
       int32_t s2 = env_step(c, eps, u, ar, cls + mo, cr ? cr + mo : NULL,
                             Q + (shared ? 0 : (size_t)i * K), sum, start[i], &s[i], &ep_step[i],
-                            &episode[i], &reward[i], &done[i], &action[i]);
+                            &episode[i], &reward[i], &done[i], &action[i], ret_acc ? &st : NULL);
       if (i < trace_n) {
         size_t o = (size_t)k * trace_n + i;
-        tr_s[o] = s2;
-        tr_a[o] = action[i];
-        tr_r[o] = reward[i];
-        tr_d[o] = done[i];
+        if (s2 >= 0) {
+          tr_s[o] = s2;
+          tr_a[o] = action[i];
+          tr_r[o] = reward[i];
+          tr_d[o] = done[i];
+        } else { /* budget used up: the env stays where it is */
+          tr_s[o] = s[i];
+          tr_a[o] = 0;
+          tr_r[o] = 0.0f;
+          tr_d[o] = 0;
+        }
       }
     }
     if (shared) tree_apply(sum, Q);
@@ -577,7 +619,7 @@ int orc_run_range(const orc_config* c, int32_t lo, int32_t hi, const uint8_t* cl
       orc_explore_draw(c->seed, (uint32_t)i, t, A, &u, &ar);
       float eps = eps_at(c, tab, len, t, episode[i]);
       env_step(c, eps, u, ar, cls + mo, cr ? cr + mo : NULL, Q + (size_t)i * K, NULL, start[i],
-               &s[i], &ep_step[i], &episode[i], &reward[i], &done[i], &action[i]);
+               &s[i], &ep_step[i], &episode[i], &reward[i], &done[i], &action[i], NULL);
     }
   }
   free(tab);

@@ -68,7 +68,7 @@ class Oracle:
         lib.orc_tree_sum_bruteforce.argtypes = [vp, vp, C.c_int, C.c_int, vp]
         lib.orc_eps_table.argtypes = [vp, vp, C.c_int]
         lib.orc_run.argtypes = [vp, vp, vp, vp, vp, vp, vp, vp, vp, vp, vp, u64, i32, vp, vp, i32, vp, vp,
-                                vp, vp]
+                                vp, vp, vp, vp, vp, vp, vp]
         lib.orc_run_range.argtypes = [vp, i32, i32, vp, vp, vp, vp, vp, vp, vp, vp, vp, vp, u64, i32]
 
     @staticmethod
@@ -143,8 +143,15 @@ class Oracle:
                     episode=np.zeros(N, np.int32), reward=np.zeros(N, np.float32),
                     done=np.zeros(N, np.uint8), action=np.zeros(N, np.uint8))
 
-    def run(self, cfg, cls, cr, start, Q, st, t0, n_steps, u=None, a_rand=None, trace_n=0):
-        """Advance `st` and `Q` in place; returns the trace dict (or None)."""
+    @staticmethod
+    def new_stats(n):
+        return dict(ret_acc=np.zeros(n, np.float32), last_return=np.zeros(n, np.float32),
+                    return_sum=np.zeros(n, np.float32), last_length=np.zeros(n, np.int32),
+                    length_sum=np.zeros(n, np.int32))
+
+    def run(self, cfg, cls, cr, start, Q, st, t0, n_steps, u=None, a_rand=None, trace_n=0, stats=None):
+        """Advance `st` and `Q` (and `stats`, from new_stats) in place; returns the
+        trace dict (or None)."""
         cls = np.ascontiguousarray(cls, np.uint8)
         cr = None if cr is None else np.ascontiguousarray(cr, np.float32)
         start = np.ascontiguousarray(start, np.int32)
@@ -161,7 +168,12 @@ class Oracle:
                               self._p(st["reward"]), self._p(st["done"]), self._p(st["action"]), t0,
                               n_steps, self._p(u), self._p(a_rand), trace_n,
                               self._p(tr["s_next"]) if tr else None, self._p(tr["action"]) if tr else None,
-                              self._p(tr["reward"]) if tr else None, self._p(tr["done"]) if tr else None)
+                              self._p(tr["reward"]) if tr else None, self._p(tr["done"]) if tr else None,
+                              self._p(stats["ret_acc"]) if stats else None,
+                              self._p(stats["last_return"]) if stats else None,
+                              self._p(stats["return_sum"]) if stats else None,
+                              self._p(stats["last_length"]) if stats else None,
+                              self._p(stats["length_sum"]) if stats else None)
         assert rc == 0
         return tr
 

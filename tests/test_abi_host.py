@@ -28,9 +28,9 @@ def test_library_exports_every_declared_symbol(pycrl):
 
 
 def test_config_struct_matches_header(pycrl):
-    # 23 four-byte fields then one uint64 at an 8-byte boundary
-    assert C.sizeof(pycrl.Config) == 96
-    assert pycrl.Config.seed.offset == 88
+    # 24 four-byte fields then one uint64 at an 8-byte boundary
+    assert C.sizeof(pycrl.Config) == 104
+    assert pycrl.Config.seed.offset == 96
 
 
 def test_philox_matches_oracle_and_kat(pycrl, oracle):
@@ -54,7 +54,8 @@ def test_philox_matches_oracle_and_kat(pycrl, oracle):
 def test_create_rejects_bad_configs_without_touching_a_device(pycrl):
     lib = pycrl.load()
     bad = [dict(n_envs=0), dict(width=0), dict(n_actions=5), dict(table_mode=3), dict(max_mode=2),
-           dict(episode_len=-1), dict(reward_flags=2), dict(eps_mode=1, eps_span=0), dict(auto_reset=2)]
+           dict(episode_len=-1), dict(reward_flags=2), dict(eps_mode=1, eps_span=0), dict(auto_reset=2),
+           dict(max_episodes=-1), dict(track_returns=2)]
     for kw in bad:
         base = dict(n_envs=4, width=4, height=4)
         base.update(kw)

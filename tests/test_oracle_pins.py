@@ -544,3 +544,41 @@ def test_run_shared_table_uses_the_tree(oracle, pycrl):
         d[i] = f(f(0.001) * f(target - pre[key[i]]))
     want = (pre + oracle.tree_sum(key, d, W * H * A)).astype(np.float32)
     assert np.array_equal(Q, want)
+
+
+def test_episode_budget_and_return_accumulators(oracle, pycrl):
+    """max_episodes / return tracking (src/train.py:186-226): the accumulators
+    equal what the trace says, episode by episode, and an env that has used its
+    budget does nothing more."""
+    W, H, A, N, T, E = 6, 6, 4, 40, 400, 5
+    cls, start = pycrl.gen_maps_bernoulli(77, N, N, W, H, 0.1, 0.05)
+    cfg = pycrl.make_config(N, W, H, episode_len=23, eps0=0.4, seed=6, max_episodes=E, track_returns=1)
+    Q = np.zeros((N, W * H, A), np.float32)
+    st, stats = oracle.new_state(cfg, start), oracle.new_stats(N)
+    tr = oracle.run(cfg, cls, None, start, Q, st, 0, T, trace_n=N, stats=stats)
+    assert (st["episode"] == E).all()  # everyone finished the budget within T steps
+    f = np.float32
+    for i in range(N):
+        rets, lens, acc, n, k = [], [], f(0), 0, 0
+        while len(rets) < E:
+            acc = f(acc + tr["reward"][k, i])
+            n += 1
+            if tr["done"][k, i] or n >= 23:
+                rets.append(acc)
+                lens.append(n)
+                acc, n = f(0), 0
+            k += 1
+        assert stats["last_return"][i] == rets[-1] and stats["last_length"][i] == lens[-1]
+        tot = f(0)
+        for r in rets:
+            tot = f(tot + r)
+        assert stats["return_sum"][i] == tot and stats["length_sum"][i] == sum(lens)
+        assert stats["ret_acc"][i] == 0
+        # after the budget: idle rows, the env stays on its start cell
+        assert (tr["s_next"][k:, i] == start[i]).all() and (tr["reward"][k:, i] == 0).all()
+        assert (tr["action"][k:, i] == 0).all() and (tr["done"][k:, i] == 0).all()
+    # the frozen steps changed nothing: a run cut at the last active step gives the same tables
+    Q2 = np.zeros((N, W * H, A), np.float32)
+    st2 = oracle.new_state(cfg, start)
+    oracle.run(cfg, cls, None, start, Q2, st2, 0, 2 * T)
+    assert np.array_equal(Q, Q2) and np.array_equal(st["s"], st2["s"])
