@@ -40,6 +40,19 @@ BatchedEnvironment::State BatchedEnvironment::state() const {
   return st;
 }
 
+BatchedEnvironment::EpisodeStats BatchedEnvironment::episodeStats() const {
+  EpisodeStats st;
+  const size_t n = (size_t)cfg.n_envs;
+  st.last_return.resize(n);
+  st.return_sum.resize(n);
+  st.last_length.resize(n);
+  st.length_sum.resize(n);
+  check(crl_get_episode_stats(engine, st.last_return.data(), st.last_length.data(), st.return_sum.data(),
+                              st.length_sum.data()),
+        "episodeStats");
+  return st;
+}
+
 std::vector<float> BatchedEnvironment::qTable(int table) const {
   std::vector<float> q((size_t)numStates() * numActions());
   check(crl_q_get(engine, table, q.data()), "qTable");

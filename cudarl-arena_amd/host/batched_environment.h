@@ -39,6 +39,12 @@ class BatchedEnvironment {
     std::vector<uint8_t> done, action;
   };
   State state() const;
+  // needs config().track_returns
+  struct EpisodeStats {
+    std::vector<float> last_return, return_sum;
+    std::vector<int32_t> last_length, length_sum;
+  };
+  EpisodeStats episodeStats() const;
   std::vector<float> qTable(int table = 0) const;
   void setQTable(int table, const std::vector<float>& q);
   uint64_t stepCount() const;

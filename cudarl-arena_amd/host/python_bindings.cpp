@@ -11,6 +11,7 @@
 
 #include "batched_environment.h"
 #include "environment_bridge.h"
+#include "npy.h"
 #include "q_learning.h"
 
 namespace py = pybind11;
@@ -258,6 +259,28 @@ PYBIND11_MODULE(cudarl_core, m) {
         t->deleter = view_deleter;
         return py::reinterpret_steal<py::object>(PyCapsule_New(t, "dltensor", capsule_destructor));
       });
+
+  // QTableAgent.save / load (src/train.py:150-168): float64 (W, H, A) .npy files indexed
+  // [x, y, a]; the table handed in / out is the engine's fp32 [(y*W + x)*A + a]
+  m.def("save_agent_npy",
+        [](const std::string& path, py::array_t<float, py::array::c_style | py::array::forcecast> q, int width,
+           int height, int actions) {
+          crl_npy::save_agent(path, std::vector<float>(q.data(), q.data() + q.size()), width, height, actions);
+        },
+        py::arg("path"), py::arg("q"), py::arg("width"), py::arg("height"), py::arg("actions") = 4);
+  m.def("load_agent_npy",
+        [](const std::string& path, int width, int height, int actions) {
+          const std::vector<float> q = crl_npy::load_agent(path, width, height, actions);
+          py::array_t<float> a({(py::ssize_t)(width * height), (py::ssize_t)actions});
+          std::memcpy(a.mutable_data(), q.data(), q.size() * sizeof(float));
+          return a;
+        },
+        py::arg("path"), py::arg("width"), py::arg("height"), py::arg("actions") = 4);
+  m.def("save_table_npy",
+        [](const std::string& path, py::array_t<float, py::array::c_style | py::array::forcecast> q) {
+          std::vector<int64_t> shape(q.shape(), q.shape() + q.ndim());
+          crl_npy::save_f32(path, shape, q.data());
+        });
 
   m.attr("__version__") = "0.1.0";
 }

@@ -115,3 +115,47 @@ def test_noise_maps(pycrl):
     walls = (cls[0] == 3).reshape(H, W)
     same_right = (walls[:, 1:] == walls[:, :-1]).mean()
     assert same_right > 0.9
+
+
+def test_npy_agent_files_match_numpy(pycrl, tmp_path):
+    """QTableAgent.save / load files (src/train.py:150-168): float64 (W, H, A)
+    indexed [x, y, a], exchanged with numpy in both directions."""
+    import sys
+    sys.path.insert(0, os.path.join(ROOT, "cudarl-arena_amd", "lib"))
+    import cudarl_core
+    W, H, A = 7, 5, 4
+    rng = np.random.default_rng(0)
+    q = rng.normal(0, 1, (W * H, A)).astype(np.float32)
+    path = str(tmp_path / "agent.npy")
+    cudarl_core.save_agent_npy(path, q, W, H, A)
+    ref = np.load(path)
+    assert ref.dtype == np.float64 and ref.shape == (W, H, A)
+    for x in range(W):
+        for y in range(H):
+            assert np.array_equal(ref[x, y], q[y * W + x].astype(np.float64))
+    assert np.array_equal(cudarl_core.load_agent_npy(path, W, H, A), q)
+    # a file written by numpy, as the reference's agent.save would
+    table = rng.normal(0, 1, (W, H, A))
+    np.save(path, table)
+    got = cudarl_core.load_agent_npy(path, W, H, A)
+    assert got.dtype == np.float32 and got.shape == (W * H, A)
+    assert np.array_equal(got.reshape(H, W, A), np.transpose(table, (1, 0, 2)).astype(np.float32))
+    np.save(path, table.astype(np.float32))
+    assert np.array_equal(cudarl_core.load_agent_npy(path, W, H, A), got)
+    with pytest.raises(RuntimeError, match="Invalid Q-table size"):
+        cudarl_core.load_agent_npy(path, W + 1, H, A)
+    np.save(path, np.asfortranarray(table))
+    with pytest.raises(RuntimeError):
+        cudarl_core.load_agent_npy(path, W, H, A)
+    np.save(path, np.arange(5))
+    with pytest.raises(RuntimeError):
+        cudarl_core.load_agent_npy(path, W, H, A)
+    with pytest.raises(RuntimeError):
+        cudarl_core.load_agent_npy(str(tmp_path / "missing.npy"), W, H, A)
+    # raw fp32 tables of any shape
+    big = rng.normal(0, 1, (3, 6, 8)).astype(np.float32)
+    cudarl_core.save_table_npy(path, big)
+    back = np.load(path)
+    assert back.dtype == np.float32 and np.array_equal(back, big)
+    cudarl_core.save_table_npy(path, big[0, 0])
+    assert np.array_equal(np.load(path), big[0, 0])

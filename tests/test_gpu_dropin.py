@@ -310,3 +310,65 @@ def test_batched_environment_dlpack_views(core, gpu):
     assert hip.hipMemcpy(host.ctypes.data, t.data, host.nbytes, 2) == 0
     with pytest.raises(RuntimeError):
         core.BatchedEnvironment(4, 4, 4).dlpack("nope")
+
+
+# ---- the training driver (src/train.py as a C++ program) ----------------------------
+
+def run_train(*args):
+    import subprocess
+    exe = os.path.join(LIBDIR, "cudarl_train")
+    out = subprocess.run([exe] + [str(a) for a in args], capture_output=True, text=True, timeout=100)
+    assert out.returncode == 0, out.stderr
+    return out.stdout.splitlines()
+
+
+def test_train_cli_reproduces_the_training_log(gpu):
+    """training.log:24930-24953: mock env (the agent never moves, nothing ends an
+    episode), 10 episodes x 500 steps, then 10 evaluation episodes of 1000 steps."""
+    g = json.load(open(os.path.join(ROOT, "tests", "golden", "training_log_vector.json")))
+    lines = run_train("--mock-env", "--episodes", g["episodes"], "--max-steps", g["max_steps"],
+                      "--eval-episodes", 10)
+    ep = [l for l in lines if l.startswith("Episode ")]
+    assert len(ep) == g["episodes"]
+    for k, line in enumerate(ep):
+        assert line.startswith("Episode %d/%d | Reward: %s | Avg Reward: %s | Avg Length: 500.0 | Epsilon: %s |"
+                               % (k + 1, g["episodes"], g["episode_return"], g["episode_return"],
+                                  g["epsilon_after_episode"][k])), line
+    ev = [l for l in lines if l.startswith("Evaluation episode")]
+    assert ev == ["Evaluation episode %d: Reward = %s, Length = %d" % (i + 1, g["eval_return"], g["eval_length"])
+                  for i in range(10)]
+    assert "Evaluation results: Avg Reward = %s, Avg Length = 1000.0" % g["eval_return"] in lines
+
+
+def test_train_cli_learns_and_saves_the_reference_file(gpu, oracle, tmp_path):
+    """Default world (10x10, centre start, goal top-right), the reference's flags;
+    the saved file is the reference's float64 [x, y, a] layout and equals the
+    oracle's table for the same configuration."""
+    E, T, W, H = 200, 100, 10, 10
+    lines = run_train("--episodes", E, "--max-steps", T, "--eval-episodes", 3, "--save-agent",
+                      "--output-dir", tmp_path, "--seed", 4)
+    ev = [l for l in lines if l.startswith("Evaluation episode")]
+    assert ev == ["Evaluation episode %d: Reward = 0.92, Length = 9" % (i + 1) for i in range(3)]  # 9 moves to the goal
+    table = np.load(os.path.join(str(tmp_path), "qtable_agent.npy"))
+    assert table.dtype == np.float64 and table.shape == (W, H, 4)
+    cfg = gpu.make_config(1, W, H, map_mode=gpu.MAP_SHARED, episode_len=T, lr=0.1, gamma=0.99,
+                          eps_mode=gpu.EPS_STEP_MULT, eps0=1.0, eps_decay=0.995, eps_span=E * T + 1,
+                          max_episodes=E, track_returns=1, seed=4)
+    cls = np.zeros(W * H, np.uint8)
+    cls[W - 1] = 1
+    start = [(H // 2) * W + W // 2]
+    Q = np.zeros((1, W * H, 4), np.float32)
+    st = oracle.new_state(cfg, start)
+    oracle.run(cfg, cls, None, start, Q, st, 0, E * T)
+    assert st["episode"][0] == E
+    want = np.transpose(Q[0].reshape(H, W, 4), (1, 0, 2)).astype(np.float64)
+    assert np.array_equal(table, want)
+
+
+def test_train_cli_many_envs(gpu):
+    lines = run_train("--episodes", 50, "--max-steps", 100, "--eval-episodes", 1, "--envs", 3000, "--width", 8,
+                      "--height", 8)
+    assert any(l.startswith("Episode 50/50") for l in lines)
+    assert "Evaluation episode 1: Reward = 0.94, Length = 7" in lines  # (4,4) -> (7,0)
+    done = [l for l in lines if l.startswith("Done!")][0]
+    assert int(done.split("(")[1].split()[0]) > 3000 * 50 * 7
