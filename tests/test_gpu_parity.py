@@ -420,26 +420,58 @@ def test_step_rule_brute_force_against_float_grid(gpu, oracle):
             assert (st["s"][i], st["reward"][i], st["done"][i]) == (y * W + x, np.float32(r), d), (trial, i)
 
 
-def test_full_size_properties_config4_slice(gpu):
-    """Size-independent properties at a large N (no oracle): positions stay on
-    non-blocking cells, rewards come from the rule's value set, every table
-    entry of a never-visited (walled) cell stays zero, and two runs agree."""
-    N, W, H, steps = 1 << 17, 16, 16, 256
+def test_full_size_config4(gpu, oracle):
+    """The whole 1,048,576-env / 4 GB configuration for its 1000 steps: three
+    1024-env slices (first, middle, last) bit-exact against the oracle, and
+    size-independent properties over all envs: positions on non-blocking cells,
+    rewards from the rule's value set, counters in range, both kinds of workers used."""
+    from conftest import oracle_run_slice
+    N, W, H, steps = 1 << 20, 16, 16, 1000
     cls, start = gpu.gen_maps_bernoulli(0, N, N, W, H, 0.1, 0.02)
     cfg = gpu.make_config(N, W, H, episode_len=128, eps0=0.1, gamma=0.95, seed=0, trap_reward=-1.0)
-    outs = []
-    for _ in range(2):
-        with gpu.Engine(cfg, 0) as eng:
-            eng.set_maps(cls, start)
-            eng.run_fused(steps)
-            st = eng.get_state()
-            q = eng.q_get(0, 2048)
-        outs.append((st, q))
-    st, q = outs[0]
-    assert all(np.array_equal(outs[0][0][k], outs[1][0][k]) for k in st) and np.array_equal(q, outs[1][1])
+    slices = [(0, 1024), (N // 2 + 77, N // 2 + 77 + 1024), (N - 1024, N)]
+    with gpu.Engine(cfg, 0) as eng:
+        eng.set_maps(cls, start)
+        eng.run_fused(steps)
+        st = eng.get_state()
+        qs = [eng.q_get(lo, hi - lo) for lo, hi in slices]
+        hbm, lds = eng.fused_split()
+        info = eng.fused_kernel_info()
+    assert "fast,hbm+lds" in info["name"] and hbm + lds == N and hbm > 0 and lds > 0
+    for (lo, hi), q in zip(slices, qs):
+        Q, ost = oracle_run_slice(oracle, cfg, lo, hi, cls[lo:hi], start[lo:hi], 0, steps)
+        assert_q_close(q.reshape(Q.shape), Q)
+        for k in ("s", "ep_step", "episode", "reward", "done", "action"):
+            assert np.array_equal(st[k][lo:hi], ost[k]), (lo, k)
     here = cls[np.arange(N), st["s"]]
     assert (here < 2).all()
     assert set(np.unique(st["reward"]).tolist()) <= {np.float32(-0.01), np.float32(1.0), np.float32(-1.0)}
-    blocked = cls[:2048] >= 2
-    assert (q[blocked] == 0).all()
-    assert (st["ep_step"] < 128).all() and st["episode"].min() >= 2
+    assert (st["ep_step"] < 128).all() and st["episode"].min() >= steps // 128
+
+
+def test_full_size_config2(gpu, oracle):
+    """4096 envs, 32x32, 256-step episodes, all 10,000 steps: final tables and
+    state bit-exact against the oracle."""
+    N, W, H, steps = 4096, 32, 32, 10000
+    cls, start = gpu.gen_maps_bernoulli(0, N, N, W, H, 0.2)
+    cfg = gpu.make_config(N, W, H, episode_len=256, lr=0.1, gamma=0.99, eps0=0.1, seed=0)
+    with gpu.Engine(cfg, 0) as eng:
+        eng.set_maps(cls, start)
+        eng.run_fused(steps)
+        st, q = eng.get_state(), eng.q_get(0, N)
+    Q = np.zeros((N, W * H, 4), np.float32)
+    ost = oracle.new_state(cfg, start)
+    import ctypes as C
+    import threading
+    p = oracle._p
+    def work(lo, hi):
+        assert oracle.lib.orc_run_range(C.byref(cfg), lo, hi, p(cls), None, p(start), p(Q), p(ost["s"]),
+                                        p(ost["ep_step"]), p(ost["episode"]), p(ost["reward"]),
+                                        p(ost["done"]), p(ost["action"]), 0, steps) == 0
+    ths = [threading.Thread(target=work, args=(N * i // 8, N * (i + 1) // 8)) for i in range(8)]
+    [t.start() for t in ths]
+    [t.join() for t in ths]
+    assert_q_close(q.reshape(Q.shape), Q)
+    for k in ("s", "ep_step", "episode", "reward", "done", "action"):
+        assert np.array_equal(st[k], ost[k]), k
+    assert st["episode"].min() >= steps // 256
