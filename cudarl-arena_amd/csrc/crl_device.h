@@ -50,7 +50,7 @@ __device__ __forceinline__ void action_delta(int a, int A, int& dx, int& dy) {
 // src/environment.cu:17-48).  `cls(cell)` returns the class of a cell of this
 // env's map, `cr` its per-cell rewards (may be null when unused).
 template <class ClassOf>
-__device__ __forceinline__ void step_rule(const Rules& R, ClassOf cls, const float* __restrict__ cr,
+__device__ __forceinline__ void step_rule(const Rules& R, const ClassOf& cls, const float* __restrict__ cr,
                                           int& x, int& y, int a, float& reward, bool& hit) {
   int dx, dy;
   action_delta(a, R.A, dx, dy);

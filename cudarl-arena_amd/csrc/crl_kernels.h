@@ -108,11 +108,52 @@ struct LdsTable {  // staged into LDS for the whole launch
   __device__ __forceinline__ void store(int s, int a, float v) const { q[s * A + a] = v; }
 };
 
-// n_steps of one env.  `cls(cell)` gives the class of a cell of the env's map,
-// `cr` its per-cell rewards (or null), `tab` its table.
+// A map too large for LDS, read from global memory: the words that hold the
+// 3 x 3 cells around the env are fetched when it ARRIVES on a cell (together with
+// the table row of that cell), so that the class of the next target comes from
+// registers and a step has one memory round trip on its critical path, not two.
+struct NearMap {
+  const uint32_t* g;
+  int W, H;
+  uint32_t w0, w1, w2, w3, w4, w5;  // rows y-1, y, y+1: the words of x-1 and of x+1
+  int i0, i1, i2, i3, i4, i5;       // their word indices
+  __device__ __forceinline__ void arrive(int x, int y) {
+    const int xl = max(x - 1, 0), xr = min(x + 1, W - 1);
+    const int ya = max(y - 1, 0) * W, yb = y * W, yc = min(y + 1, H - 1) * W;
+    i0 = (ya + xl) >> 4; i1 = (ya + xr) >> 4;
+    i2 = (yb + xl) >> 4; i3 = (yb + xr) >> 4;
+    i4 = (yc + xl) >> 4; i5 = (yc + xr) >> 4;
+    w0 = g[i0]; w1 = g[i1]; w2 = g[i2]; w3 = g[i3]; w4 = g[i4]; w5 = g[i5];
+  }
+  // class of a cell at most one step away from the cell of the last arrive()
+  __device__ __forceinline__ int operator()(int cell) const {
+    const int i = cell >> 4;
+    uint32_t w = w0;
+    w = (i == i1) ? w1 : w;
+    w = (i == i2) ? w2 : w;
+    w = (i == i3) ? w3 : w;
+    w = (i == i4) ? w4 : w;
+    w = (i == i5) ? w5 : w;
+    return cell_class_of(w, cell);
+  }
+};
+
+// a map in LDS needs no such preparation
+template <class F>
+struct LdsMap {
+  F word_of;  // cell -> packed word
+  __device__ __forceinline__ void arrive(int, int) {}
+  __device__ __forceinline__ int operator()(int cell) const { return cell_class_of(word_of(cell), cell); }
+};
+template <class F>
+__device__ __forceinline__ LdsMap<F> lds_map(F f) { return LdsMap<F>{f}; }
+
+// n_steps of one env.  `cls(cell)` gives the class of a cell of the env's map
+// (cls.arrive(x, y) is called whenever the env lands on a cell), `cr` its
+// per-cell rewards (or null), `tab` its table.
 template <int A, class Table, class ClassOf>
 __device__ __forceinline__ void run_env_steps(const Rules& R, const Ptrs& P, const int env,
-                                              const uint64_t t0, const int n_steps, ClassOf cls,
+                                              const uint64_t t0, const int n_steps, ClassOf& cls,
                                               const float* __restrict__ cr, const Table tab) {
   const int start = P.start[env];
   const int sx = start % R.W, sy = start / R.W;
@@ -124,6 +165,7 @@ __device__ __forceinline__ void run_env_steps(const Rules& R, const Ptrs& P, con
   float reward = P.reward[env];  // rewritten unchanged if the env's episode budget is used up
   int action = P.action[env];
   Row<A> row = tab.load(s);
+  cls.arrive(x, y);
   Philox4 blk = explore_block(R.seed, (uint32_t)env, t0 >> 1);
   const bool track = P.ret_acc != nullptr;
   float ret = track ? P.ret_acc[env] : 0.0f;
@@ -152,7 +194,11 @@ __device__ __forceinline__ void run_env_steps(const Rules& R, const Ptrs& P, con
 
     // Q row of the new cell; when the env did not move it is the row in registers
     Row<A> row2 = row;
-    if (s2 != s0) row2 = tab.load(s2);
+    const bool ends = R.auto_reset && (done || (R.episode_len > 0 && ep_step + 1 >= R.episode_len));
+    if (s2 != s0) {
+      row2 = tab.load(s2);
+      if (!ends) cls.arrive(x, y);  // the new neighbourhood, in the shadow of the row load
+    }
     // the next step's draws depend on nothing: the Philox rounds run while the
     // row load is in flight
     if ((t & 1) == 1) blk = explore_block(R.seed, (uint32_t)env, (t + 1) >> 1);
@@ -171,7 +217,7 @@ __device__ __forceinline__ void run_env_steps(const Rules& R, const Ptrs& P, con
       P.tr_r[o] = reward;
       P.tr_d[o] = done ? 1 : 0;
     }
-    if (R.auto_reset && (done || (R.episode_len > 0 && ep_step >= R.episode_len))) {
+    if (ends) {
       if (track) record_episode(P, env, ret, ep_step);
       ret = 0.0f;
       x = sx;
@@ -180,6 +226,7 @@ __device__ __forceinline__ void run_env_steps(const Rules& R, const Ptrs& P, con
       ep_step = 0;
       episode += 1;
       row = tab.load(start);
+      cls.arrive(x, y);
       if (start == s0) row = row_set(row, a, qn);  // the value just written, from registers
     } else {
       s = s2;
@@ -297,14 +344,19 @@ __global__ __launch_bounds__(256) void k_fused_per_env(const Rules R, const Ptrs
   for (int chunk = blockIdx.x; chunk < n_chunks; chunk += gridDim.x) {
     const int env = chunk * bdim + tid;
     if (env >= P.N) continue;
-    const uint32_t* gmap = P.map + (P.map_shared ? 0 : (size_t)env * P.map_words);
-    auto cls = [&](int cell) -> int {
-      const uint32_t word = (MAP == 1) ? lds[cell >> 4] : gmap[cell >> 4];
-      return cell_class_of(word, cell);
-    };
     const float* cr =
         P.cell_reward ? P.cell_reward + (P.map_shared ? 0 : (size_t)env * P.S) : nullptr;
-    run_env_steps<A>(R, P, env, t0, n_steps, cls, cr, GlobalTable<A>{P.Q + (size_t)env * P.S * A});
+    const GlobalTable<A> tab{P.Q + (size_t)env * P.S * A};
+    if (MAP == 1) {
+      auto cls = lds_map([&](int cell) -> uint32_t { return lds[cell >> 4]; });
+      run_env_steps<A>(R, P, env, t0, n_steps, cls, cr, tab);
+    } else {
+      NearMap cls{};
+      cls.g = P.map + (P.map_shared ? 0 : (size_t)env * P.map_words);
+      cls.W = R.W;
+      cls.H = R.H;
+      run_env_steps<A>(R, P, env, t0, n_steps, cls, cr, tab);
+    }
   }
 }
 
@@ -341,7 +393,7 @@ __global__ __launch_bounds__(LDSW ? 320 : 256) void k_fused_tickets(const Rules 
   const unsigned take = lds_worker ? 1u : 2u;
   const size_t table = P.S * A;  // floats per table
   auto mapw = [&](int word) -> uint32_t { return my_map[word * 64 + lane]; };
-  auto cls = [&](int cell) -> int { return cell_class_of(my_map[(cell >> 4) * 64 + lane], cell); };
+  auto cls = lds_map([&](int cell) -> uint32_t { return my_map[(cell >> 4) * 64 + lane]; });
 
   while (true) {
     unsigned base = 0;
