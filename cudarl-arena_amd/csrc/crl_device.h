@@ -116,6 +116,15 @@ __device__ __forceinline__ Row<4> load_row<4>(const float* __restrict__ p) { ret
 template <>
 __device__ __forceinline__ Row<8> load_row<8>(const float* __restrict__ p) { return load_row8(p); }
 
+// Keeps the optimiser from merging a conditionally loaded row with another one
+// (which would make the conditional load wait for the other row first).
+__device__ __forceinline__ void row_opaque(Row<4>& r) {
+  asm volatile("" : "+v"(r.q0), "+v"(r.q1), "+v"(r.q2), "+v"(r.q3));
+}
+__device__ __forceinline__ void row_opaque(Row<8>& r) {
+  asm volatile("" : "+v"(r.q0), "+v"(r.q1), "+v"(r.q2), "+v"(r.q3), "+v"(r.q4), "+v"(r.q5), "+v"(r.q6), "+v"(r.q7));
+}
+
 // lowest index wins ties (src/q_learning.cu:200-206: strict >)
 __device__ __forceinline__ void amax_step(float v, int i, float& bv, int& bi) {
   const bool gt = v > bv;

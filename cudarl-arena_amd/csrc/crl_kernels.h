@@ -125,6 +125,11 @@ struct NearMap {
     i4 = (yc + xl) >> 4; i5 = (yc + xr) >> 4;
     w0 = g[i0]; w1 = g[i1]; w2 = g[i2]; w3 = g[i3]; w4 = g[i4]; w5 = g[i5];
   }
+  // the words of the last arrive() have landed (a loop entered with loads still
+  // in flight waits for every outstanding memory operation on each iteration)
+  __device__ __forceinline__ void settle() {
+    asm volatile("" : "+v"(w0), "+v"(w1), "+v"(w2), "+v"(w3), "+v"(w4), "+v"(w5));
+  }
   // class of a cell at most one step away from the cell of the last arrive()
   __device__ __forceinline__ int operator()(int cell) const {
     const int i = cell >> 4;
@@ -143,6 +148,7 @@ template <class F>
 struct LdsMap {
   F word_of;  // cell -> packed word
   __device__ __forceinline__ void arrive(int, int) {}
+  __device__ __forceinline__ void settle() {}
   __device__ __forceinline__ int operator()(int cell) const { return cell_class_of(word_of(cell), cell); }
 };
 template <class F>
@@ -152,9 +158,14 @@ __device__ __forceinline__ LdsMap<F> lds_map(F f) { return LdsMap<F>{f}; }
 // (cls.arrive(x, y) is called whenever the env lands on a cell), `cr` its
 // per-cell rewards (or null), `tab` its table.
 template <int A, class Table, class ClassOf>
-__device__ __forceinline__ void run_env_steps(const Rules& R, const Ptrs& P, const int env,
+__device__ __forceinline__ void run_env_steps(const Rules& R_in, const Ptrs& P, const int env,
                                               const uint64_t t0, const int n_steps, ClassOf& cls,
                                               const float* __restrict__ cr, const Table tab) {
+  // The class rewards as plain register values.  As loads from the kernel's
+  // argument block, "cell reward or class reward" is turned into one load through
+  // a selected pointer, which needs the class rewards copied to scratch memory.
+  Rules R = R_in;
+  asm volatile("" : "+s"(R.step_reward), "+s"(R.goal_reward), "+s"(R.trap_reward));
   const int start = P.start[env];
   const int sx = start % R.W, sy = start / R.W;
   int s = P.s[env];
@@ -169,6 +180,10 @@ __device__ __forceinline__ void run_env_steps(const Rules& R, const Ptrs& P, con
   Philox4 blk = explore_block(R.seed, (uint32_t)env, t0 >> 1);
   const bool track = P.ret_acc != nullptr;
   float ret = track ? P.ret_acc[env] : 0.0f;
+  // nothing loaded above is still in flight when the loop starts
+  row_opaque(row);
+  cls.settle();
+  asm volatile("" : "+v"(ep_step), "+v"(episode), "+v"(reward), "+v"(action), "+v"(ret));
 
   for (int k = 0; k < n_steps; ++k) {
     if (R.max_episodes > 0 && episode >= R.max_episodes) {
@@ -192,20 +207,27 @@ __device__ __forceinline__ void run_env_steps(const Rules& R, const Ptrs& P, con
     const int s2 = y * R.W + x;
     done = hit || (!R.auto_reset && done);
 
-    // Q row of the new cell; when the env did not move it is the row in registers
+    // Q row of the new cell; when the env did not move it is the row in registers.
+    // An env whose episode ends with this step also needs the row and the
+    // neighbourhood of its start cell: known now, so everything is requested in
+    // one go and a step has one memory round trip
     Row<A> row2 = row;
     const bool ends = R.auto_reset && (done || (R.episode_len > 0 && ep_step + 1 >= R.episode_len));
-    if (s2 != s0) {
-      row2 = tab.load(s2);
-      if (!ends) cls.arrive(x, y);  // the new neighbourhood, in the shadow of the row load
+    if (s2 != s0) row2 = tab.load(s2);
+    Row<A> row_start{};
+    if (ends) {
+      row_start = tab.load(start);
+      cls.arrive(sx, sy);
+    } else if (s2 != s0) {
+      cls.arrive(x, y);
     }
     // the next step's draws depend on nothing: the Philox rounds run while the
-    // row load is in flight
+    // loads are in flight
     if ((t & 1) == 1) blk = explore_block(R.seed, (uint32_t)env, (t + 1) >> 1);
+    row_opaque(row_start);
     const float m = row_max(row2, done, R.max_mode);
     const float qn = td_value(row_get(row, a), reward, m, R.lr, R.gamma);
     tab.store(s0, a, qn);
-    if (s2 == s0) row2 = row_set(row2, a, qn);
 
     ep_step += 1;
     action = a;
@@ -217,21 +239,15 @@ __device__ __forceinline__ void run_env_steps(const Rules& R, const Ptrs& P, con
       P.tr_r[o] = reward;
       P.tr_d[o] = done ? 1 : 0;
     }
-    if (ends) {
-      if (track) record_episode(P, env, ret, ep_step);
-      ret = 0.0f;
-      x = sx;
-      y = sy;
-      s = start;
-      ep_step = 0;
-      episode += 1;
-      row = tab.load(start);
-      cls.arrive(x, y);
-      if (start == s0) row = row_set(row, a, qn);  // the value just written, from registers
-    } else {
-      s = s2;
-      row = row2;
-    }
+    if (ends && track) record_episode(P, env, ret, ep_step);
+    // the cell to act from next, with the value just written patched in from registers
+    s = ends ? start : s2;
+    row = row_set(ends ? row_start : row2, s == s0 ? a : -1, qn);
+    x = ends ? sx : x;
+    y = ends ? sy : y;
+    ret = ends ? 0.0f : ret;
+    ep_step = ends ? 0 : ep_step;
+    episode += ends ? 1 : 0;
   }
 
   P.s[env] = s;
@@ -271,6 +287,13 @@ __device__ __forceinline__ void run_env_fast(const Rules& R, const Ptrs& P, cons
   bool odd = (t0 & 1) != 0;
   uint64_t next_block = (t0 >> 1) + 1;
 
+  // everything loaded above has arrived before the loop starts: a value still in
+  // flight at the loop's entry makes the loop's first instruction wait for ALL
+  // outstanding memory operations on every iteration, the previous step's store
+  // included
+  row_opaque(row);
+  asm volatile("" : "+v"(ep_step), "+v"(episode));
+
   for (int k = 0; k < n_steps; ++k) {
     const uint32_t w0 = odd ? blk.w2 : blk.w0;
     const uint32_t w1 = odd ? blk.w3 : blk.w1;
@@ -293,29 +316,30 @@ __device__ __forceinline__ void run_env_fast(const Rules& R, const Ptrs& P, cons
     reward = hit ? r_goal : (cls == kTrap ? r_trap : r_step);
 
     // the row of the cell the env stands on next; an env that stayed reads its own
-    // row again (still the pre-update values: the write below comes later)
+    // row again (still the pre-update values: the write below comes later).  An env
+    // whose episode ends with this step needs its start cell's row instead: that is
+    // known before any row arrives, so both loads are in flight together
     Row<A> row2 = tab.load(s2);
-    if (odd) blk = explore_block(R.seed, (uint32_t)env, next_block++);  // in the load's shadow
+    ep_step += 1;
+    const bool ends = hit || (T > 0 && ep_step >= T);
+    Row<A> row_start{};
+    if (ends) row_start = tab.load(start);
+    if (odd) blk = explore_block(R.seed, (uint32_t)env, next_block++);  // in the loads' shadow
+    row_opaque(row_start);
     const float m = row_max(row2, hit, 0);
     const float qn = td_value(row_get(row, a), reward, m, lr, gamma);
     tab.store(s, a, qn);
-    row2 = row_set(row2, s2 == s ? a : -1, qn);
 
+    // the cell to act from next, with the value just written patched in from registers
+    const int s_next = ends ? start : s2;
+    row = row_set(ends ? row_start : row2, s_next == s ? a : -1, qn);
+    x = ends ? sx : x;
+    y = ends ? sy : y;
+    ep_step = ends ? 0 : ep_step;
+    episode += ends ? 1 : 0;
+    s = s_next;
     action = a;
-    ep_step += 1;
     odd = !odd;
-    if (hit || (T > 0 && ep_step >= T)) {
-      row = tab.load(start);
-      row = row_set(row, start == s ? a : -1, qn);  // the value just written, from registers
-      x = sx;
-      y = sy;
-      s = start;
-      ep_step = 0;
-      episode += 1;
-    } else {
-      s = s2;
-      row = row2;
-    }
   }
 
   P.s[env] = s;
@@ -367,9 +391,9 @@ __global__ __launch_bounds__(256) void k_fused_per_env(const Rules R, const Ptrs
 // how many bytes of their tables - are live on the chip at once: few enough and
 // the rows an env keeps returning to are still in the last-level cache.
 //
-// Waves 0-3 of a workgroup step 64 envs each against tables in HBM / the caches,
-// and spend most of their time waiting for one row per step.  With LDSW a fifth
-// wave uses the idle issue slots and the LDS: it stages the WHOLE tables of 32
+// All waves of a workgroup but the last step 64 envs each against tables in HBM /
+// the caches, and spend most of their time waiting for one row per step.  With
+// LDSW the last wave uses the idle issue slots and the LDS: it stages the WHOLE tables of 32
 // envs into LDS, steps them there and writes the tables back.  The split between
 // the two kinds follows their speed; which worker steps an env does not change
 // its results.  FAST selects the folded loop (run_env_fast).
@@ -382,13 +406,13 @@ __global__ __launch_bounds__(LDSW ? 320 : 256) void k_fused_tickets(const Rules 
                                                                      unsigned* __restrict__ ticket,
                                                                      const int tab_stride) {
   extern __shared__ uint32_t lds[];
-  constexpr int kWaves = LDSW ? 5 : 4;
+  const int n_waves = (int)(blockDim.x >> 6);  // with LDSW the last one works on LDS tables
   const int lane = threadIdx.x & 63;
   const int wave = threadIdx.x >> 6;
   uint32_t* my_map = lds + wave * (P.map_words * 64);  // [word][lane]
-  float* tabs = reinterpret_cast<float*>(lds + kWaves * (P.map_words * 64));
+  float* tabs = reinterpret_cast<float*>(lds + n_waves * (P.map_words * 64));
   const unsigned n_tickets = (unsigned)((P.N + kTicketEnvs - 1) / kTicketEnvs);
-  const bool lds_worker = LDSW && wave == 4;
+  const bool lds_worker = LDSW && wave == n_waves - 1;
   const int cap = lds_worker ? kTicketEnvs : 64;
   const unsigned take = lds_worker ? 1u : 2u;
   const size_t table = P.S * A;  // floats per table
@@ -430,22 +454,25 @@ __global__ __launch_bounds__(LDSW ? 320 : 256) void k_fused_tickets(const Rules 
       const float4* g4 = reinterpret_cast<const float4*>(P.Q + (size_t)env0 * table);
       const int t4 = (int)(table / 4);
       const int total4 = n_here * t4;
-      for (int i0 = 0; i0 < total4; i0 += 64 * 8) {
-        float4 v[8];  // eight loads in flight per lane
-#pragma unroll
-        for (int u = 0; u < 8; ++u) {
-          const int i = i0 + u * 64 + lane;
-          if (i < total4) v[u] = g4[i];
-        }
-#pragma unroll
-        for (int u = 0; u < 8; ++u) {
-          const int i = i0 + u * 64 + lane;
-          if (i < total4) {
-            const int e = i / t4, o = i - e * t4;
-            reinterpret_cast<float4*>(tabs + e * tab_stride)[o] = v[u];
-          }
-        }
+      auto put = [&](int i, const float4 v) {
+        const int e = i / t4, o = i - e * t4;
+        reinterpret_cast<float4*>(tabs + e * tab_stride)[o] = v;
+      };
+      int i0 = 0;
+      for (; i0 + 64 * 8 <= total4; i0 += 64 * 8) {  // eight loads in flight per lane
+        const int i = i0 + lane;
+        const float4 v0 = g4[i], v1 = g4[i + 64], v2 = g4[i + 128], v3 = g4[i + 192];
+        const float4 v4 = g4[i + 256], v5 = g4[i + 320], v6 = g4[i + 384], v7 = g4[i + 448];
+        put(i, v0);
+        put(i + 64, v1);
+        put(i + 128, v2);
+        put(i + 192, v3);
+        put(i + 256, v4);
+        put(i + 320, v5);
+        put(i + 384, v6);
+        put(i + 448, v7);
       }
+      for (int i = i0 + lane; i < total4; i += 64) put(i, g4[i]);
       __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
       __builtin_amdgcn_wave_barrier();
       if (live) {
