@@ -84,6 +84,47 @@ __device__ __forceinline__ void step_rule(const Rules& R, const ClassOf& cls, co
   reward = r;
 }
 
+// Move codes: what each action does from one cell, 2 bits per action -
+//   0 the env moves, 1 it moves onto the goal, 2 a trap (stays, trap reward),
+//   3 blocked by a wall or by the edge of the grid (stays, step reward)
+// - which is the class of the target cell, or 3 outside the grid.  Valid for the
+// rule that tests the goal on the target cell (src/kernels.cu:34-66).  With the
+// codes of the cell it stands on in a register, an env's next cell follows from
+// its action without a map lookup or a bounds test.
+// `word_of(i)` returns word i of the env's packed class map.
+template <int A, class WordOf>
+__device__ __forceinline__ uint32_t moves_of_cell(WordOf word_of, int W, int H, int x, int y, int s) {
+  // all map words are asked for before the first one is looked at (a target
+  // outside the grid reads the env's own cell instead, and the result is dropped)
+  uint32_t word[A];
+#pragma unroll
+  for (int a = 0; a < A; ++a) {
+    int dx, dy;
+    action_delta(a, A, dx, dy);  // constants once the loop is unrolled
+    const bool in = (dx == 0 || (unsigned)(x + dx) < (unsigned)W) &&
+                    (dy == 0 || (unsigned)(y + dy) < (unsigned)H);
+    const int tgt = in ? s + dy * W + dx : s;
+    word[a] = word_of(tgt >> 4);
+  }
+#pragma unroll
+  for (int a = 0; a < A; ++a) asm volatile("" : "+v"(word[a]));  // keeps the reads unconditional
+  uint32_t mv = 0;
+#pragma unroll
+  for (int a = 0; a < A; ++a) {
+    int dx, dy;
+    action_delta(a, A, dx, dy);
+    const bool in = (dx == 0 || (unsigned)(x + dx) < (unsigned)W) &&
+                    (dy == 0 || (unsigned)(y + dy) < (unsigned)H);
+    const int tgt = s + dy * W + dx;
+    const uint32_t code = in ? (uint32_t)cell_class_of(word[a], tgt) : (uint32_t)kWall;
+    mv |= code << (2 * a);
+  }
+  return mv;
+}
+// packed move codes: 16/A cells per 32-bit word
+template <int A>
+__device__ __forceinline__ constexpr int move_cells_per_word() { return 16 / A; }
+
 // One table row in registers.  Named scalars passed BY VALUE: an element picked
 // by a run-time action index must compile to a chain of selects.  Through a
 // reference the optimiser folds "select of two loads" into one indexed load

@@ -71,6 +71,7 @@ struct crl_engine {
   int N = 0, W = 0, H = 0, A = 0;
   size_t S = 0, K = 0;
   int n_maps = 0, n_tables = 0, map_words = 0;
+  int mv_words = 0;  // words of move codes per map; 0: no move codes are kept
   uint64_t t = 0;
   long resident_envs = 0;  // 0 = automatic
   int fused_variant = 0;   // 0 = automatic, 1 = plain, 2 = hybrid (when it fits)
@@ -81,6 +82,7 @@ struct crl_engine {
   DevBuf<float> reward;
   DevBuf<uint8_t> done, action;
   DevBuf<uint32_t> map;
+  DevBuf<uint32_t> moves;  // move codes derived from map, for the folded fused loop
   DevBuf<float> cell_reward;
   DevBuf<float> Q;
   DevBuf<float> eps_tab;
@@ -149,6 +151,7 @@ struct crl_engine {
     P.done = done.p;
     P.action = action.p;
     P.map = map.p;
+    P.moves = moves.p;
     P.cell_reward = (cfg.reward_flags & CRL_REWARD_CELLS) ? cell_reward.p : nullptr;
     P.Q = Q.p;
     P.eps_tab = eps_tab.p;
@@ -170,6 +173,7 @@ struct crl_engine {
     P.len_sum = len_sum.p;
     P.N = N;
     P.map_words = map_words;
+    P.mv_words = mv_words;
     P.map_shared = cfg.map_mode == CRL_MAP_SHARED;
     P.table_shared = cfg.table_mode == CRL_TABLE_SHARED;
     P.S = S;
@@ -205,6 +209,7 @@ struct FusedPlan {
   bool tickets;    // per-env maps in LDS: waves draw env ranges from a ticket counter
   bool hybrid;     // ... with a fifth wave per workgroup that steps envs whose tables it holds in LDS
   bool fast;       // the folded loop for the common configuration
+  bool moves;      // ... whose table waves read pre-built move codes from LDS
   int tab_stride;  // floats between two tables in LDS
 };
 
@@ -233,8 +238,8 @@ FusedPlan plan_fused(const crl_engine* e) {
   }
   // Envs live on the chip at once.  A worker steps its envs for all n steps
   // before it takes the next ones, so a smaller grid means fewer tables in
-  // flight: when all tables together exceed the last-level cache, keep as many
-  // in flight as fit into it (but never less than one wave per SIMD of the chip).
+  // flight: when all tables together exceed what the last-level cache holds well,
+  // keep that many bytes in flight (but never less than three waves per compute unit).
   long resident = e->resident_envs;
   if (resident <= 0) {
     const size_t table_bytes = e->K * sizeof(float);
@@ -250,37 +255,42 @@ FusedPlan plan_fused(const crl_engine* e) {
     p.fast = c.eps_mode == CRL_EPS_FIXED && c.reward_flags == 0 && c.goal_mode == CRL_GOAL_ON_TARGET &&
              c.auto_reset == 1 && c.max_mode == CRL_MAX_TRUE && e->trace_n == 0 && e->sup_n == 0 &&
              c.max_episodes == 0 && c.track_returns == 0;
+    p.fast = p.fast && e->mv_words > 0;
     // Hybrid workgroups when 32 whole tables (padded by one row against bank
-    // conflicts) and five waves' maps fit into LDS.
+    // conflicts), the LDS wave's maps and at least one table wave's maps fit into
+    // LDS.  One workgroup per compute unit (the LDS holds no second one); the envs
+    // in flight on HBM tables set how many 64-env waves work beside the LDS wave.
     p.tab_stride = (int)e->K + 4;
     const size_t map_lds = (size_t)e->map_words * 64 * 4;
-    const size_t hybrid_lds = 5 * map_lds + (size_t)crl::kTicketEnvs * p.tab_stride * 4;
-    const bool fits = e->K % 4 == 0 && hybrid_lds <= kLdsPerWorkgroup;
-    p.hybrid = fits && (e->fused_variant == 2 || (e->fused_variant == 0 && e->N >= kHybridMinEnvs));
+    const size_t mv_lds = (size_t)e->mv_words * 64 * 4;
+    const size_t lds_wave = p.fast ? (size_t)e->mv_words * crl::kTicketEnvs * 4 : map_lds;
+    const size_t tables_lds = (size_t)crl::kTicketEnvs * p.tab_stride * 4;
     const long tickets = (e->N + crl::kTicketEnvs - 1) / crl::kTicketEnvs;
+    const bool fits = e->K % 4 == 0 && map_lds + lds_wave + tables_lds <= kLdsPerWorkgroup;
+    p.hybrid = fits && (e->fused_variant == 2 || (e->fused_variant == 0 && e->N >= kHybridMinEnvs));
     if (p.hybrid) {
-      // one workgroup per compute unit (the LDS holds no second one); the envs in
-      // flight on HBM tables set how many 64-env waves work beside the LDS wave
       p.grid = (int)std::min<long>(kComputeUnits, (tickets + 8) / 9);
-      const long hbm_waves = std::min<long>(4, std::max<long>(1, resident / (64L * p.grid)));
+      long hbm_waves = std::min<long>(4, std::max<long>(1, resident / (64L * p.grid)));
+      while (hbm_waves * map_lds + lds_wave + tables_lds > kLdsPerWorkgroup) --hbm_waves;
       p.block = 64 * ((int)hbm_waves + 1);
-      p.lds = (hbm_waves + 1) * map_lds + (size_t)crl::kTicketEnvs * p.tab_stride * 4;
-    } else if (tickets / 2 < 4 * 256) {
-      // fewer 64-env workers than SIMDs on the chip: one-wave workgroups spread
-      // them over the compute units instead of packing four per unit
-      p.block = 64;
-      p.lds = map_lds;
-      p.grid = (int)std::min<long>(std::max<long>(1, resident / 64), (tickets + 1) / 2);
-    } else if (resident <= 4L * 64 * kComputeUnits) {
-      // at most four waves per compute unit: spread them over all units
-      const long waves = std::max<long>(1, resident / (64L * kComputeUnits));
-      p.block = 64 * (int)waves;
-      p.lds = waves * map_lds;
-      p.grid = (int)std::min<long>(kComputeUnits, (tickets + 2 * waves - 1) / (2 * waves));
+      p.lds = hbm_waves * map_lds + lds_wave + tables_lds;
     } else {
-      p.block = 256;
-      p.lds = 4 * map_lds;
-      p.grid = (int)std::min<long>(std::max<long>(1, resident / 256), (tickets + 7) / 8);
+      long waves = 4;
+      if (tickets / 2 < 4 * kComputeUnits) {
+        // fewer 64-env workers than SIMDs on the chip: one-wave workgroups spread
+        // them over the compute units instead of packing four per unit
+        waves = 1;
+        p.grid = (int)std::min<long>(std::max<long>(1, resident / 64), (tickets + 1) / 2);
+      } else if (resident <= 4L * 64 * kComputeUnits) {
+        // at most four waves per compute unit: spread them over all units
+        waves = std::max<long>(1, resident / (64L * kComputeUnits));
+        p.grid = (int)std::min<long>(kComputeUnits, (tickets + 2 * waves - 1) / (2 * waves));
+      } else {
+        p.grid = (int)std::min<long>(std::max<long>(1, resident / 256), (tickets + 7) / 8);
+      }
+      p.block = 64 * (int)waves;
+      p.moves = p.fast && waves * mv_lds <= kLdsPerWorkgroup;
+      p.lds = waves * (p.moves ? mv_lds : map_lds);
     }
   }
   static const char* names[2][3] = {
@@ -306,14 +316,20 @@ void launch_fused_a(const crl_engine* e, const FusedPlan& p, uint64_t t0, int n)
     hipLaunchKernelGGL(crl::k_fill_u32, dim3(1), dim3(64), 0, e->stream, e->ticket.p, 0u, 3);
     const dim3 g(p.grid), b(p.block);
     unsigned* tk = e->ticket.p;
+#define CRL_LAUNCH_TICKETS(FAST, LDSW, MOVES)                                                       \
+  hipLaunchKernelGGL((crl::k_fused_tickets<A, FAST, LDSW, MOVES>), g, b, p.lds, e->stream, R, P, t0, n, \
+                     tk, p.tab_stride)
     if (p.fast && p.hybrid)
-      hipLaunchKernelGGL((crl::k_fused_tickets<A, true, true>), g, b, p.lds, e->stream, R, P, t0, n, tk, p.tab_stride);
+      CRL_LAUNCH_TICKETS(true, true, false);
+    else if (p.fast && p.moves)
+      CRL_LAUNCH_TICKETS(true, false, true);
     else if (p.fast)
-      hipLaunchKernelGGL((crl::k_fused_tickets<A, true, false>), g, b, p.lds, e->stream, R, P, t0, n, tk, p.tab_stride);
+      CRL_LAUNCH_TICKETS(true, false, false);
     else if (p.hybrid)
-      hipLaunchKernelGGL((crl::k_fused_tickets<A, false, true>), g, b, p.lds, e->stream, R, P, t0, n, tk, p.tab_stride);
+      CRL_LAUNCH_TICKETS(false, true, false);
     else
-      hipLaunchKernelGGL((crl::k_fused_tickets<A, false, false>), g, b, p.lds, e->stream, R, P, t0, n, tk, p.tab_stride);
+      CRL_LAUNCH_TICKETS(false, false, false);
+#undef CRL_LAUNCH_TICKETS
     return;
   }
   switch (p.map_kind) {
@@ -464,6 +480,21 @@ int check_engine(const crl_engine* e) {
   return CRL_OK;
 }
 
+// move codes of maps [first, first + count) from the class maps on the device
+int build_moves(crl_engine* e, int first, int count) {
+  if (e->mv_words == 0 || count <= 0) return CRL_OK;
+  const size_t threads = (size_t)count * e->mv_words;
+  const dim3 g((unsigned)((threads + 255) / 256)), b(256);
+  if (e->A == 4)
+    hipLaunchKernelGGL(crl::k_build_moves<4>, g, b, 0, e->stream, e->map.p, e->map_words, e->W, e->H,
+                       e->mv_words, first, count, e->moves.p);
+  else
+    hipLaunchKernelGGL(crl::k_build_moves<8>, g, b, 0, e->stream, e->map.p, e->map_words, e->W, e->H,
+                       e->mv_words, first, count, e->moves.p);
+  HIP_TRY(hipGetLastError());
+  return CRL_OK;
+}
+
 int upload_maps(crl_engine* e) {
   std::vector<uint32_t> packed((size_t)e->n_maps * e->map_words, 0u);
   for (int m = 0; m < e->n_maps; ++m)
@@ -475,6 +506,8 @@ int upload_maps(crl_engine* e) {
     HIP_TRY(hipMemcpyAsync(e->cell_reward.p, e->h_cell_reward.data(),
                            e->h_cell_reward.size() * sizeof(float), hipMemcpyHostToDevice,
                            e->stream));
+  const int rc = build_moves(e, 0, e->n_maps);
+  if (rc) return rc;
   HIP_TRY(hipStreamSynchronize(e->stream));
   return CRL_OK;
 }
@@ -537,6 +570,12 @@ int crl_create(const crl_config* cfg, int device, crl_engine** out) {
   acc(e->done.alloc(N));
   acc(e->action.alloc(N));
   acc(e->map.alloc((size_t)e->n_maps * e->map_words));
+  // move codes for the folded fused loop: per-env maps that the ticket kernel stages in LDS
+  if (cfg->map_mode != CRL_MAP_SHARED && (size_t)e->map_words * 4 * 64 <= (size_t)kLdsMapLimitBytes) {
+    const size_t cells_per_word = 16 / (size_t)e->A;
+    e->mv_words = (int)((e->S + cells_per_word - 1) / cells_per_word);
+    acc(e->moves.alloc((size_t)e->n_maps * e->mv_words));
+  }
   if (cells) acc(e->cell_reward.alloc((size_t)e->n_maps * e->S));
   acc(e->Q.alloc((size_t)e->n_tables * e->K));
   acc(e->eps_tab.alloc(eps.size()));
@@ -692,6 +731,8 @@ int crl_set_cell(crl_engine* e, int32_t map_index, int32_t cell, int32_t cell_cl
   for (size_t j = 0; j < 16 && ((size_t)(cell >> 4) << 4) + j < e->S; ++j)
     packed |= (uint32_t)(e->h_class[first + j] & 3u) << (2 * j);
   HIP_TRY(hipMemcpyAsync(e->map.p + word, &packed, 4, hipMemcpyHostToDevice, e->stream));
+  rc = build_moves(e, map_index, 1);  // the neighbours' codes name this cell
+  if (rc) return rc;
   if (e->cfg.reward_flags & CRL_REWARD_CELLS) {
     e->h_cell_reward[at] = cell_reward;
     HIP_TRY(hipMemcpyAsync(e->cell_reward.p + at, &cell_reward, 4, hipMemcpyHostToDevice, e->stream));
@@ -841,10 +882,12 @@ int crl_run_fused(crl_engine* e, int32_t n_steps) {
       if (e->ticket.ensure(3) != hipSuccess) return fail(CRL_E_ALLOC, "ticket counter allocation failed");
       if (!e->hybrid_opt_in) {
         const void* fns[] = {
-            reinterpret_cast<const void*>(&crl::k_fused_tickets<4, true, true>),
-            reinterpret_cast<const void*>(&crl::k_fused_tickets<4, false, true>),
-            reinterpret_cast<const void*>(&crl::k_fused_tickets<8, true, true>),
-            reinterpret_cast<const void*>(&crl::k_fused_tickets<8, false, true>)};
+            reinterpret_cast<const void*>(&crl::k_fused_tickets<4, true, true, false>),
+            reinterpret_cast<const void*>(&crl::k_fused_tickets<4, false, true, false>),
+            reinterpret_cast<const void*>(&crl::k_fused_tickets<4, true, false, true>),
+            reinterpret_cast<const void*>(&crl::k_fused_tickets<8, true, true, false>),
+            reinterpret_cast<const void*>(&crl::k_fused_tickets<8, false, true, false>),
+            reinterpret_cast<const void*>(&crl::k_fused_tickets<8, true, false, true>)};
         for (const void* fn : fns)
           HIP_TRY(hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, (int)kLdsPerWorkgroup));
         e->hybrid_opt_in = true;

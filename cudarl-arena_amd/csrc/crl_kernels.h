@@ -4,6 +4,7 @@
 //   s, ep_step, episode : int32    reward : fp32    done, action : uint8
 //   start               : int32 cell index
 //   map                 : 2 bits per cell, 16 cells per uint32, map_words per map
+//   moves               : 2 bits per (cell, action), derived from map (per-env maps only)
 //   cell_reward         : fp32 per cell (optional)
 //   Q                   : fp32 [table][s][a], one table per env or one shared
 //
@@ -24,6 +25,7 @@ struct Ptrs {
   uint8_t* done;
   uint8_t* action;
   const uint32_t* map;
+  const uint32_t* moves;  // packed move codes of every cell, mv_words per map (or null)
   const float* cell_reward;
   float* Q;
   const float* eps_tab;
@@ -48,6 +50,7 @@ struct Ptrs {
   // geometry
   int N;
   int map_words;   // uint32 words per map
+  int mv_words;    // uint32 words of move codes per map
   int map_shared;  // 1: one map for all envs
   int table_shared;  // 1: one table for all envs
   size_t S;        // cells per map
@@ -259,40 +262,64 @@ __device__ __forceinline__ void run_env_steps(const Rules& R_in, const Ptrs& P, 
   P.action[env] = (uint8_t)action;
 }
 
+// Where the folded loop gets the move codes of a cell from.
+// Pre-built codes staged in LDS, word-interleaved over the wave's lanes:
+template <int A>
+struct MovesLds {
+  const uint32_t* base;  // the lane's first word
+  int stride;            // words between two consecutive words of one env
+  __device__ __forceinline__ uint32_t at(int s, int, int) const {
+    constexpr int kCells = move_cells_per_word<A>();
+    return base[(s / kCells) * stride] >> ((s % kCells) * 2 * A);
+  }
+};
+// Derived from the class map in LDS when the codes of all lanes do not fit: one
+// map word per action, asked for while the table row is in flight.
+template <int A>
+struct MovesFromMap {
+  const uint32_t* base;  // the lane's first map word, words 64 apart
+  int W, H;
+  __device__ __forceinline__ uint32_t at(int s, int x, int y) const {
+    return moves_of_cell<A>([&](int word) -> uint32_t { return base[word * 64]; }, W, H, x, y, s);
+  }
+};
+
 // The same loop for the common configuration, with everything that is fixed
 // there folded away: fixed epsilon, class rewards (no per-cell array), goal test
 // on the target cell, auto-reset, true max, no trace and no supplied stream.
 // Fewer live scalars and no optional branches: about half the instructions of
 // the general loop, which matters because a wave that waits for one row per
 // step is also issue-bound on the arithmetic between two rows.
-// `mapw(i)` returns word i of the env's packed map.
-template <int A, class Table, class MapWord>
+// Between the arrival of one row and the request for the next lie only the
+// argmax, the draw and one shift of the cell's move codes; the codes of the next
+// cell, the Philox rounds and the bookkeeping run while the row is in flight.
+template <int A, class Table, class Moves>
 __device__ __forceinline__ void run_env_fast(const Rules& R, const Ptrs& P, const int env,
-                                             const uint64_t t0, const int n_steps, MapWord mapw,
+                                             const uint64_t t0, const int n_steps, const Moves moves,
                                              const Table tab) {
-  const int W = R.W, H = R.H, T = R.episode_len;
+  const int W = R.W, T = R.episode_len;
   const float eps = R.eps0, lr = R.lr, gamma = R.gamma;
   const float r_step = R.step_reward, r_goal = R.goal_reward, r_trap = R.trap_reward;
-  const int start = P.start[env];
+  int start = P.start[env];
   const int sx = start % W, sy = start / W;
   int s = P.s[env];
-  int x = s % W, y = s / W;
+  int x = s % W, y = s / W;  // only followed when the move codes are derived from the map
   int ep_step = P.ep_step[env];
   int episode = P.episode[env];
   float reward = 0.0f;
   int action = 0;
   bool hit = false;
   Row<A> row = tab.load(s);
+  uint32_t mv = moves.at(s, x, y);
   Philox4 blk = explore_block(R.seed, (uint32_t)env, t0 >> 1);
   bool odd = (t0 & 1) != 0;
   uint64_t next_block = (t0 >> 1) + 1;
-
   // everything loaded above has arrived before the loop starts: a value still in
   // flight at the loop's entry makes the loop's first instruction wait for ALL
   // outstanding memory operations on every iteration, the previous step's store
   // included
   row_opaque(row);
-  asm volatile("" : "+v"(ep_step), "+v"(episode));
+  asm volatile("" : "+v"(ep_step), "+v"(episode), "+v"(mv), "+v"(start), "+v"(s));
 
   for (int k = 0; k < n_steps; ++k) {
     const uint32_t w0 = odd ? blk.w2 : blk.w0;
@@ -301,40 +328,37 @@ __device__ __forceinline__ void run_env_fast(const Rules& R, const Ptrs& P, cons
     const int greedy = row_argmax(row);
     const int a = (u01(w0) < eps) ? (int)below(w1, (uint32_t)A) : greedy;
 
+    const uint32_t code = (mv >> (2 * a)) & 3u;
+    const bool moved = code < (uint32_t)kTrap;
     int dx, dy;
     action_delta(a, A, dx, dy);
-    const int nx = x + dx, ny = y + dy;
-    const bool in = (unsigned)nx < (unsigned)W && (unsigned)ny < (unsigned)H;
-    const int tgt = in ? ny * W + nx : s;  // out of bounds: look at the own cell, result unused
-    const int looked = cell_class_of(mapw(tgt >> 4), tgt);
-    const int cls = in ? looked : kFree;
-    const bool moved = in && cls < kTrap;
-    x = moved ? nx : x;
-    y = moved ? ny : y;
-    const int s2 = moved ? tgt : s;
-    hit = cls == kGoal;
-    reward = hit ? r_goal : (cls == kTrap ? r_trap : r_step);
+    dx = moved ? dx : 0;
+    dy = moved ? dy : 0;
+    const int s2 = s + __mul24(dy, W) + dx;
+    hit = code == (uint32_t)kGoal;
+    reward = hit ? r_goal : (code == (uint32_t)kTrap ? r_trap : r_step);
 
-    // the row of the cell the env stands on next; an env that stayed reads its own
-    // row again (still the pre-update values: the write below comes later).  An env
-    // whose episode ends with this step needs its start cell's row instead: that is
-    // known before any row arrives, so both loads are in flight together
-    Row<A> row2 = tab.load(s2);
+    // Two rows are asked for together: the one of the cell the move ends on (for
+    // the TD target) and the one of the cell the env acts from next - the same
+    // cell, and the same cache line, unless the episode ends with this step and the
+    // env restarts.  No branch, and a restart costs no second round trip.  An env
+    // that stays where it is reads its own row again (the pre-update values: the
+    // write below comes later).
     ep_step += 1;
     const bool ends = hit || (T > 0 && ep_step >= T);
-    Row<A> row_start{};
-    if (ends) row_start = tab.load(start);
+    const int s_next = ends ? start : s2;
+    const Row<A> row2 = tab.load(s2);
+    const Row<A> row_next = tab.load(s_next);
+    x = ends ? sx : x + dx;
+    y = ends ? sy : y + dy;
+    mv = moves.at(s_next, x, y);
     if (odd) blk = explore_block(R.seed, (uint32_t)env, next_block++);  // in the loads' shadow
-    row_opaque(row_start);
     const float m = row_max(row2, hit, 0);
     const float qn = td_value(row_get(row, a), reward, m, lr, gamma);
     tab.store(s, a, qn);
 
     // the cell to act from next, with the value just written patched in from registers
-    const int s_next = ends ? start : s2;
-    row = row_set(ends ? row_start : row2, s_next == s ? a : -1, qn);
-    x = ends ? sx : x;
-    y = ends ? sy : y;
+    row = row_set(row_next, s_next == s ? a : -1, qn);
     ep_step = ends ? 0 : ep_step;
     episode += ends ? 1 : 0;
     s = s_next;
@@ -393,13 +417,28 @@ __global__ __launch_bounds__(256) void k_fused_per_env(const Rules R, const Ptrs
 //
 // All waves of a workgroup but the last step 64 envs each against tables in HBM /
 // the caches, and spend most of their time waiting for one row per step.  With
-// LDSW the last wave uses the idle issue slots and the LDS: it stages the WHOLE tables of 32
-// envs into LDS, steps them there and writes the tables back.  The split between
-// the two kinds follows their speed; which worker steps an env does not change
-// its results.  FAST selects the folded loop (run_env_fast).
+// LDSW the last wave uses the idle issue slots and the LDS: it stages the WHOLE
+// tables of 32 envs into LDS, steps them there and writes the tables back.  The
+// split between the two kinds follows their speed; which worker steps an env does
+// not change its results.
+//
+// FAST selects the folded loop (run_env_fast), which works on move codes: the
+// LDS wave always stages the pre-built codes of its envs; the table waves stage
+// them too with MOVES, and otherwise stage the (four times smaller) class maps
+// and derive the codes while their row loads are in flight.
 constexpr int kTicketEnvs = 32;
 
-template <int A, bool FAST, bool LDSW>
+// `count` envs' words (`wpe` per env, contiguous in HBM) into [word][lane]
+__device__ __forceinline__ void stage_words(const uint32_t* __restrict__ src, const int count,
+                                            const int wpe, const int stride, uint32_t* dst,
+                                            const int lane) {
+  for (int i = lane; i < count * wpe; i += 64) {
+    const int e = i / wpe, w = i - e * wpe;
+    dst[w * stride + e] = src[i];
+  }
+}
+
+template <int A, bool FAST, bool LDSW, bool MOVES>
 __global__ __launch_bounds__(LDSW ? 320 : 256) void k_fused_tickets(const Rules R, const Ptrs P,
                                                                      const uint64_t t0,
                                                                      const int n_steps,
@@ -409,15 +448,18 @@ __global__ __launch_bounds__(LDSW ? 320 : 256) void k_fused_tickets(const Rules 
   const int n_waves = (int)(blockDim.x >> 6);  // with LDSW the last one works on LDS tables
   const int lane = threadIdx.x & 63;
   const int wave = threadIdx.x >> 6;
-  uint32_t* my_map = lds + wave * (P.map_words * 64);  // [word][lane]
-  float* tabs = reinterpret_cast<float*>(lds + n_waves * (P.map_words * 64));
-  const unsigned n_tickets = (unsigned)((P.N + kTicketEnvs - 1) / kTicketEnvs);
   const bool lds_worker = LDSW && wave == n_waves - 1;
+  // LDS: one slice per table wave, the LDS wave's slice, the tables
+  constexpr bool kTableMoves = FAST && MOVES;
+  const int slice = (kTableMoves ? P.mv_words : P.map_words) * 64;
+  const int lds_slice = !LDSW ? 0 : FAST ? P.mv_words * kTicketEnvs : P.map_words * 64;
+  uint32_t* my_words = lds + wave * slice;  // (the LDS wave is the last one)
+  float* tabs = reinterpret_cast<float*>(lds + (n_waves - 1) * slice + lds_slice);
+  const unsigned n_tickets = (unsigned)((P.N + kTicketEnvs - 1) / kTicketEnvs);
   const int cap = lds_worker ? kTicketEnvs : 64;
   const unsigned take = lds_worker ? 1u : 2u;
   const size_t table = P.S * A;  // floats per table
-  auto mapw = [&](int word) -> uint32_t { return my_map[word * 64 + lane]; };
-  auto cls = lds_map([&](int cell) -> uint32_t { return my_map[(cell >> 4) * 64 + lane]; });
+  auto cls = lds_map([&](int cell) -> uint32_t { return my_words[(cell >> 4) * 64 + lane]; });
 
   while (true) {
     unsigned base = 0;
@@ -432,11 +474,11 @@ __global__ __launch_bounds__(LDSW ? 320 : 256) void k_fused_tickets(const Rules 
 
     // this worker's maps: contiguous in HBM, transposed into [word][lane]
     __builtin_amdgcn_wave_barrier();
-    const uint32_t* src = P.map + (size_t)env0 * P.map_words;
-    for (int i = lane; i < n_here * P.map_words; i += 64) {
-      const int e = i / P.map_words, w = i - e * P.map_words;
-      my_map[w * 64 + e] = src[i];
-    }
+    const bool codes = FAST && (MOVES || lds_worker);
+    if (codes)
+      stage_words(P.moves + (size_t)env0 * P.mv_words, n_here, P.mv_words, cap, my_words, lane);
+    else
+      stage_words(P.map + (size_t)env0 * P.map_words, n_here, P.map_words, 64, my_words, lane);
     const float* cr = P.cell_reward ? P.cell_reward + (size_t)env * P.S : nullptr;
 
     if (!lds_worker) {
@@ -444,8 +486,10 @@ __global__ __launch_bounds__(LDSW ? 320 : 256) void k_fused_tickets(const Rules 
       __builtin_amdgcn_wave_barrier();
       if (live) {
         const GlobalTable<A> tab{P.Q + (size_t)env * table};
-        if (FAST)
-          run_env_fast<A>(R, P, env, t0, n_steps, mapw, tab);
+        if (kTableMoves)
+          run_env_fast<A>(R, P, env, t0, n_steps, MovesLds<A>{my_words + lane, 64}, tab);
+        else if (FAST)
+          run_env_fast<A>(R, P, env, t0, n_steps, MovesFromMap<A>{my_words + lane, R.W, R.H}, tab);
         else
           run_env_steps<A>(R, P, env, t0, n_steps, cls, cr, tab);
       }
@@ -478,7 +522,7 @@ __global__ __launch_bounds__(LDSW ? 320 : 256) void k_fused_tickets(const Rules 
       if (live) {
         const LdsTable<A> tab{tabs + lane * tab_stride};
         if (FAST)
-          run_env_fast<A>(R, P, env, t0, n_steps, mapw, tab);
+          run_env_fast<A>(R, P, env, t0, n_steps, MovesLds<A>{my_words + lane, kTicketEnvs}, tab);
         else
           run_env_steps<A>(R, P, env, t0, n_steps, cls, cr, tab);
       }
@@ -750,6 +794,30 @@ __global__ __launch_bounds__(256) void k_shared_act(const Rules R, const Ptrs P,
     ReduceLds& L = *reinterpret_cast<ReduceLds*>(lds_raw);
     reduce_block(L, G, blockIdx.x, my_key, my_delta, live, handoff);
   }
+}
+
+// Move codes of maps [first, first + count) from their class maps: one thread per
+// word of codes.
+template <int A>
+__global__ __launch_bounds__(256) void k_build_moves(const uint32_t* __restrict__ map,
+                                                      const int map_words, const int W, const int H,
+                                                      const int mv_words, const int first,
+                                                      const int count, uint32_t* __restrict__ moves) {
+  constexpr int kCells = move_cells_per_word<A>();
+  const size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (i >= (size_t)count * mv_words) return;
+  const int m = first + (int)(i / mv_words), w = (int)(i % mv_words);
+  const uint32_t* g = map + (size_t)m * map_words;
+  uint32_t out = 0;
+#pragma unroll
+  for (int j = 0; j < kCells; ++j) {
+    const int c = w * kCells + j;
+    if (c < W * H) {
+      const uint32_t mv = moves_of_cell<A>([&](int word) -> uint32_t { return g[word]; }, W, H, c % W, c / W, c);
+      out |= mv << (j * 2 * A);
+    }
+  }
+  moves[(size_t)m * mv_words + w] = out;
 }
 
 __global__ void k_fill_u32(unsigned* p, const unsigned v, const int n) {

@@ -143,6 +143,68 @@ def test_fused_fast_loop_matches_oracle(gpu, oracle, variant, N, W, H, T, steps,
     assert st["episode"].max() >= 1
 
 
+@pytest.mark.parametrize("variant,resident", [(1, 0), (1, 192), (2, 0)])
+@pytest.mark.parametrize("N,W,H,A", [(2500, 16, 16, 8), (300, 9, 6, 8), (2100, 7, 5, 4), (130, 33, 31, 4)])
+def test_fused_fast_loop_move_codes(gpu, oracle, variant, resident, N, W, H, A):
+    """The folded loop works on per-cell move codes (what each action does from a
+    cell) instead of map lookups and bounds tests: pre-built codes staged in LDS
+    (plain kernel, LDS wave of the hybrid one) or derived from the class map
+    (table waves of the hybrid one), with 4 and 8 actions, on grids whose width is
+    no multiple of the 16 cells of a map word, with walls, traps and goals on the
+    edges."""
+    cls, start = gpu.gen_maps_bernoulli(43, N, N, W, H, 0.2, 0.05)
+    cfg = gpu.make_config(N, W, H, n_actions=A, episode_len=37, eps0=0.3, gamma=0.9, seed=23, trap_reward=-0.5)
+    S, steps = W * H, 150
+    with gpu.Engine(cfg, 0) as eng:
+        eng.set_maps(cls, start)
+        eng.set_fused_variant(variant)
+        eng.set_resident_envs(resident)
+        info = eng.fused_kernel_info()
+        assert "fast" in info["name"], info
+        eng.run_fused(steps)
+        q, st = eng.q_get(0, N), eng.get_state()
+    Q = np.zeros((N, S, A), np.float32)
+    ost = oracle.new_state(cfg, start)
+    oracle.run(cfg, cls, None, start, Q, ost, 0, steps)
+    for k in ("s", "ep_step", "episode", "reward", "done", "action"):
+        assert np.array_equal(st[k], ost[k]), k
+    assert_q_close(q.reshape(N, S, A), Q)
+    assert st["episode"].max() >= 1
+
+
+@pytest.mark.parametrize("variant", [1, 2])
+def test_fused_fast_loop_after_set_cell(gpu, oracle, variant):
+    """crl_set_cell changes one cell of one map: the move codes of its neighbours
+    follow, and the folded loop then agrees with the oracle on the edited maps."""
+    N, W, H, steps = 2200, 16, 16, 120
+    cls, start = gpu.gen_maps_bernoulli(47, N, N, W, H, 0.1, 0.02)
+    cfg = gpu.make_config(N, W, H, episode_len=50, eps0=0.2, gamma=0.95, seed=29)
+    cls = cls.reshape(N, W * H).copy()
+    edits = [(0, 17, gpu.CELL_WALL), (5, 200, gpu.CELL_GOAL), (2199, 34, gpu.CELL_TRAP), (77, 255, gpu.CELL_FREE),
+             (77, 0, gpu.CELL_WALL)]
+    with gpu.Engine(cfg, 0) as eng:
+        eng.set_maps(cls, start)
+        eng.set_fused_variant(variant)
+        eng.run_fused(steps)
+        for m, c, k in edits:
+            if c == start[m]:
+                continue
+            eng.set_cell(m, c, k)
+        eng.run_fused(steps)
+        assert "fast" in eng.fused_kernel_info()["name"]
+        q, st = eng.q_get(0, N), eng.get_state()
+    Q = np.zeros((N, W * H, 4), np.float32)
+    ost = oracle.new_state(cfg, start)
+    oracle.run(cfg, cls, None, start, Q, ost, 0, steps)
+    for m, c, k in edits:
+        if c != start[m]:
+            cls[m, c] = k
+    oracle.run(cfg, cls, None, start, Q, ost, steps, steps)
+    for k in ("s", "ep_step", "episode", "reward", "done", "action"):
+        assert np.array_equal(st[k], ost[k]), k
+    assert_q_close(q.reshape(N, W * H, 4), Q)
+
+
 def test_fused_large_map_global_path(gpu, oracle):
     """Maps too large for LDS are read from global memory (config 5 shape: 8
     actions, value-noise walls, per-cell rewards, linear epsilon)."""
