@@ -269,8 +269,9 @@ struct MovesLds {
   const uint32_t* base;  // the lane's first word
   int stride;            // words between two consecutive words of one env
   __device__ __forceinline__ uint32_t at(int s, int, int) const {
-    constexpr int kCells = move_cells_per_word<A>();
-    return base[(s / kCells) * stride] >> ((s % kCells) * 2 * A);
+    constexpr unsigned kCells = (unsigned)move_cells_per_word<A>();
+    const unsigned c = (unsigned)s;  // cell indices are never negative: shifts, not signed division
+    return base[(c / kCells) * (unsigned)stride] >> ((c % kCells) * 2u * A);
   }
 };
 // Derived from the class map in LDS when the codes of all lanes do not fit: one
@@ -293,12 +294,22 @@ struct MovesFromMap {
 // Between the arrival of one row and the request for the next lie only the
 // argmax, the draw and one shift of the cell's move codes; the codes of the next
 // cell, the Philox rounds and the bookkeeping run while the row is in flight.
-template <int A, class Table, class Moves>
+//
+// PAIR: lanes l and l + 32 of the wave step the SAME env (a wave that can hold
+// only 32 envs, because their tables fill the LDS, has half its lanes to spare).
+// Both do everything twice - same addresses, same values - except the Philox
+// rounds, the most expensive stretch of a step that waits for no memory: one
+// lane computes the block of the next two steps, the other the block after, and
+// they swap, so the rounds run every fourth step instead of every second.
+template <int A, bool PAIR, class Table, class Moves>
 __device__ __forceinline__ void run_env_fast(const Rules& R, const Ptrs& P, const int env,
                                              const uint64_t t0, const int n_steps, const Moves moves,
                                              const Table tab) {
   const int W = R.W, T = R.episode_len;
-  const float eps = R.eps0, lr = R.lr, gamma = R.gamma;
+  const float lr = R.lr, gamma = R.gamma;
+  // u01(w) < eps  <=>  (w >> 8) < eps * 2^24, both sides exact: an integer compare
+  const float scaled = ceilf(R.eps0 * 16777216.0f);
+  const uint32_t explore_below = !(scaled > 0.0f) ? 0u : scaled >= 16777216.0f ? (1u << 24) : (uint32_t)scaled;
   const float r_step = R.step_reward, r_goal = R.goal_reward, r_trap = R.trap_reward;
   int start = P.start[env];
   const int sx = start % W, sy = start / W;
@@ -311,9 +322,33 @@ __device__ __forceinline__ void run_env_fast(const Rules& R, const Ptrs& P, cons
   bool hit = false;
   Row<A> row = tab.load(s);
   uint32_t mv = moves.at(s, x, y);
-  Philox4 blk = explore_block(R.seed, (uint32_t)env, t0 >> 1);
+  const int lane = (int)__lane_id();
+  const bool upper = PAIR && lane >= 32;
+  // own block, and (PAIR) the partner lane's: {blk, nxt} = the next two blocks
+  auto two_blocks = [&](uint64_t b, Philox4& first, Philox4& second) {
+    const Philox4 own = explore_block(R.seed, (uint32_t)env, b + (upper ? 1 : 0));
+    Philox4 other;
+    other.w0 = (uint32_t)__shfl((int)own.w0, lane ^ 32);
+    other.w1 = (uint32_t)__shfl((int)own.w1, lane ^ 32);
+    other.w2 = (uint32_t)__shfl((int)own.w2, lane ^ 32);
+    other.w3 = (uint32_t)__shfl((int)own.w3, lane ^ 32);
+    first.w0 = upper ? other.w0 : own.w0;
+    first.w1 = upper ? other.w1 : own.w1;
+    first.w2 = upper ? other.w2 : own.w2;
+    first.w3 = upper ? other.w3 : own.w3;
+    second.w0 = upper ? own.w0 : other.w0;
+    second.w1 = upper ? own.w1 : other.w1;
+    second.w2 = upper ? own.w2 : other.w2;
+    second.w3 = upper ? own.w3 : other.w3;
+  };
+  Philox4 blk, nxt{};
+  bool have_nxt = PAIR;
+  uint64_t next_block = (t0 >> 1) + (PAIR ? 2 : 1);
+  if (PAIR)
+    two_blocks(t0 >> 1, blk, nxt);
+  else
+    blk = explore_block(R.seed, (uint32_t)env, t0 >> 1);
   bool odd = (t0 & 1) != 0;
-  uint64_t next_block = (t0 >> 1) + 1;
   // everything loaded above has arrived before the loop starts: a value still in
   // flight at the loop's entry makes the loop's first instruction wait for ALL
   // outstanding memory operations on every iteration, the previous step's store
@@ -326,7 +361,7 @@ __device__ __forceinline__ void run_env_fast(const Rules& R, const Ptrs& P, cons
     const uint32_t w1 = odd ? blk.w3 : blk.w1;
     // both candidates are computed and one is selected: cheaper than a divergent branch
     const int greedy = row_argmax(row);
-    const int a = (u01(w0) < eps) ? (int)below(w1, (uint32_t)A) : greedy;
+    const int a = ((w0 >> 8) < explore_below) ? (int)below(w1, (uint32_t)A) : greedy;
 
     const uint32_t code = (mv >> (2 * a)) & 3u;
     const bool moved = code < (uint32_t)kTrap;
@@ -352,7 +387,18 @@ __device__ __forceinline__ void run_env_fast(const Rules& R, const Ptrs& P, cons
     x = ends ? sx : x + dx;
     y = ends ? sy : y + dy;
     mv = moves.at(s_next, x, y);
-    if (odd) blk = explore_block(R.seed, (uint32_t)env, next_block++);  // in the loads' shadow
+    if (odd) {  // in the loads' shadow
+      if (!PAIR) {
+        blk = explore_block(R.seed, (uint32_t)env, next_block++);
+      } else if (have_nxt) {
+        blk = nxt;
+        have_nxt = false;
+      } else {
+        two_blocks(next_block, blk, nxt);
+        next_block += 2;
+        have_nxt = true;
+      }
+    }
     const float m = row_max(row2, hit, 0);
     const float qn = td_value(row_get(row, a), reward, m, lr, gamma);
     tab.store(s, a, qn);
@@ -487,9 +533,9 @@ __global__ __launch_bounds__(LDSW ? 320 : 256) void k_fused_tickets(const Rules 
       if (live) {
         const GlobalTable<A> tab{P.Q + (size_t)env * table};
         if (kTableMoves)
-          run_env_fast<A>(R, P, env, t0, n_steps, MovesLds<A>{my_words + lane, 64}, tab);
+          run_env_fast<A, false>(R, P, env, t0, n_steps, MovesLds<A>{my_words + lane, 64}, tab);
         else if (FAST)
-          run_env_fast<A>(R, P, env, t0, n_steps, MovesFromMap<A>{my_words + lane, R.W, R.H}, tab);
+          run_env_fast<A, false>(R, P, env, t0, n_steps, MovesFromMap<A>{my_words + lane, R.W, R.H}, tab);
         else
           run_env_steps<A>(R, P, env, t0, n_steps, cls, cr, tab);
       }
@@ -519,20 +565,34 @@ __global__ __launch_bounds__(LDSW ? 320 : 256) void k_fused_tickets(const Rules 
       for (int i = i0 + lane; i < total4; i += 64) put(i, g4[i]);
       __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
       __builtin_amdgcn_wave_barrier();
-      if (live) {
+      if (FAST) {
+        // lanes l and l + 32 both step env l of the ticket
+        const int l = lane & (kTicketEnvs - 1);
+        if (l < n_here) {
+          const LdsTable<A> tab{tabs + l * tab_stride};
+          run_env_fast<A, true>(R, P, env0 + l, t0, n_steps, MovesLds<A>{my_words + l, kTicketEnvs}, tab);
+        }
+      } else if (live) {
         const LdsTable<A> tab{tabs + lane * tab_stride};
-        if (FAST)
-          run_env_fast<A>(R, P, env, t0, n_steps, MovesLds<A>{my_words + lane, kTicketEnvs}, tab);
-        else
-          run_env_steps<A>(R, P, env, t0, n_steps, cls, cr, tab);
+        run_env_steps<A>(R, P, env, t0, n_steps, cls, cr, tab);
       }
       __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
       __builtin_amdgcn_wave_barrier();
       float4* o4 = reinterpret_cast<float4*>(P.Q + (size_t)env0 * table);
-      for (int i = lane; i < total4; i += 64) {
+      auto get = [&](int i) -> float4 {
         const int e = i / t4, o = i - e * t4;
-        o4[i] = reinterpret_cast<const float4*>(tabs + e * tab_stride)[o];
+        return reinterpret_cast<const float4*>(tabs + e * tab_stride)[o];
+      };
+      int j0 = 0;
+      for (; j0 + 64 * 4 <= total4; j0 += 64 * 4) {
+        const int i = j0 + lane;
+        const float4 v0 = get(i), v1 = get(i + 64), v2 = get(i + 128), v3 = get(i + 192);
+        o4[i] = v0;
+        o4[i + 64] = v1;
+        o4[i + 128] = v2;
+        o4[i + 192] = v3;
       }
+      for (int i = j0 + lane; i < total4; i += 64) o4[i] = get(i);
     }
   }
 }
