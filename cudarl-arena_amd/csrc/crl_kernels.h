@@ -778,6 +778,7 @@ __global__ __launch_bounds__(256) void k_shared_act(const Rules R, const Ptrs P,
   bool live = env < P.N;
   // the env's cell is fetched while the map streams into LDS
   const int s_in = live ? P.s[env] : 0;
+  if (REDUCE) reduce_block_clear(*reinterpret_cast<ReduceLds*>(lds_raw), G);
   if (MAP == 1) {
     for (int i = tid; i < P.map_words; i += blockDim.x) lds_map[i] = P.map[i];
     __syncthreads();
@@ -803,6 +804,19 @@ __global__ __launch_bounds__(256) void k_shared_act(const Rules R, const Ptrs P,
     const int s0 = s_in;
     int x = s0 % R.W, y = s0 / R.W;
     const Row<A> row = load_row<A>(Q + (size_t)s0 * A);
+    // The TD target needs the largest value of the row of the cell the move ends
+    // on - one of the A neighbours, or this cell.  All of them are asked for now,
+    // with the env's own row, instead of one more dependent round trip once the
+    // action is known (the table is small and shared: these reads hit the caches).
+    float nb_max[A];
+#pragma unroll
+    for (int i = 0; i < A; ++i) {
+      int dx, dy;
+      action_delta(i, A, dx, dy);
+      const bool in = (unsigned)(x + dx) < (unsigned)R.W && (unsigned)(y + dy) < (unsigned)R.H;
+      const int cell = in ? s0 + dy * R.W + dx : s0;
+      nb_max[i] = row_max(load_row<A>(Q + (size_t)cell * A), false, 0);
+    }
     Draw d = pick_draw(explore_block(R.seed, (uint32_t)env, t >> 1), t, A);
     if (P.u_sup && t >= P.sup_t0 && t - P.sup_t0 < (uint64_t)P.sup_n) {
       const size_t o = (size_t)(t - P.sup_t0) * P.N + env;
@@ -817,8 +831,11 @@ __global__ __launch_bounds__(256) void k_shared_act(const Rules R, const Ptrs P,
     step_rule(R, cls, cr, x, y, a, reward, hit);
     const int s2 = y * R.W + x;
     const bool done = hit || (!R.auto_reset && P.done[env] != 0);
-    const Row<A> row2 = load_row<A>(Q + (size_t)s2 * A);
-    const float m = row_max(row2, done, R.max_mode);
+    float m = row_max(row, false, 0);  // the env stayed where it was
+#pragma unroll
+    for (int i = 0; i < A; ++i) m = (s2 != s0 && a == i) ? nb_max[i] : m;
+    if (R.max_mode == 1) m = fmaxf(0.0f, m);
+    m = done ? 0.0f : m;
     my_key = s0 * A + a;
     my_delta = td_delta(row_get(row, a), reward, m, R.lr, R.gamma);
     key[env] = my_key;

@@ -24,8 +24,8 @@ namespace crl {
 constexpr int kBlockSamples = 256;   // level 0
 constexpr int kGroupBlocks = 16;     // level 1
 constexpr int kOwnKeys = 64;         // keys per owner workgroup
-constexpr int kSlotCap = 15;         // block sums one block can hand one owner
-constexpr int kHandoffRecs = 16;     // one 128-byte hand-off cell: header {count, -} + 15 records
+constexpr int kSlotCap = 8;          // block sums one block can hand one owner
+constexpr int kHandoffRecs = 8;      // one 64-byte hand-off cell of 8 records {key slot | count << 8, sum}
 constexpr int kSlotOverflow = 255;   // count value: read the block's raw samples instead
 constexpr int kDenseKeys = 16384;    // keys the dense LDS table of pass 1 can hold
 constexpr int kTileBlocks = 256;     // blocks per LDS tile of pass 2
@@ -57,8 +57,19 @@ struct ReduceLds {
   int handed[256];            // block sums handed to each owner so far
 };
 
-// Pass 1 for one block.  All 256 threads of the workgroup call it with their
-// sample (valid = false: no sample / no delta).  key < K <= kDenseKeys.
+// Clears the block's LDS state.  Needs no sample, so a kernel calls it first and
+// lets it overlap with the loads that produce the samples; reduce_block() has the
+// barrier that orders it before the first use.
+__device__ __forceinline__ void reduce_block_clear(ReduceLds& L, const ReduceGeom G) {
+  const int tid = threadIdx.x;
+  uint4* seen4 = reinterpret_cast<uint4*>(L.seen);
+  for (int i = tid; i < kDenseKeys / 16; i += kBlockSamples) seen4[i] = make_uint4(0, 0, 0, 0);
+  if (tid < (1 << G.own_shift)) L.handed[tid] = 0;
+}
+
+// Pass 1 for one block, after reduce_block_clear().  All 256 threads of the
+// workgroup call it with their sample (valid = false: no sample / no delta).
+// key < K <= kDenseKeys.
 __device__ __forceinline__ void reduce_block(ReduceLds& L, const ReduceGeom G, const int block,
                                              const int key, const float delta, const bool valid,
                                              uint2* __restrict__ handoff) {
@@ -66,10 +77,6 @@ __device__ __forceinline__ void reduce_block(ReduceLds& L, const ReduceGeom G, c
   const int lane = tid & 63;
   const int wave = tid >> 6;
   const int n_own = 1 << G.own_shift;
-
-  uint4* seen4 = reinterpret_cast<uint4*>(L.seen);
-  for (int i = tid; i < kDenseKeys / 16; i += kBlockSamples) seen4[i] = make_uint4(0, 0, 0, 0);
-  if (tid < n_own) L.handed[tid] = 0;
 
   // lanes of this wave that hold the same key
   unsigned long long peers = __ballot(valid);
@@ -82,18 +89,32 @@ __device__ __forceinline__ void reduce_block(ReduceLds& L, const ReduceGeom G, c
   const int owner = owner_of(key, G.own_shift);
   bool first = false;
   int slot = 0;
+  // The waves take turns below (a key's running sum passes from wave to wave), so
+  // what can be done before a wave's turn is done here, by all waves at once: a
+  // leader fetches the deltas of its first eight samples, itself included.  Absent
+  // ones are +0.0f, which leaves a sum that started from +0.0f unchanged.
+  constexpr int kAhead = 8;
+  unsigned long long rest = leader ? peers : 0ull;
+  float ahead[kAhead];
+#pragma unroll
+  for (int i = 0; i < kAhead; ++i) {
+    const int j = rest ? __builtin_ctzll(rest) : lane;
+    const float dj = __shfl(delta, j);
+    ahead[i] = rest ? dj : 0.0f;
+    rest &= rest - 1ull;
+  }
   __syncthreads();
 
   for (int w = 0; w < 4; ++w) {
     if (wave == w) {
       float acc = 0.0f;
-      unsigned long long rest = 0ull;
       if (leader) {
         first = L.seen[key] == 0;
         acc = first ? 0.0f : L.run[key];
-        rest = peers;
       }
-      while (__ballot(rest != 0ull) != 0ull) {
+#pragma unroll
+      for (int i = 0; i < kAhead; ++i) acc = acc + ahead[i];  // lane order = sample order
+      while (__ballot(rest != 0ull) != 0ull) {  // the rare key with more than eight samples in a wave
         const int j = rest ? __builtin_ctzll(rest) : lane;
         const float dj = __shfl(delta, j);
         if (rest) acc = acc + dj;  // lane order = sample order
@@ -108,17 +129,19 @@ __device__ __forceinline__ void reduce_block(ReduceLds& L, const ReduceGeom G, c
     __syncthreads();
   }
 
-  // hand-off cell of (owner, block): record 0 is the header, so that the owner
-  // gets count and records with one independent 128-byte read
+  // hand-off cell of (owner, block): 64 bytes that the owner gets with one
+  // independent read; record 0 also carries the count (0: nothing for this owner)
   if (leader && first && slot < kSlotCap) {
-    const size_t at = ((size_t)owner * G.n_blocks + block) * kHandoffRecs + 1 + slot;
-    handoff[at] = make_uint2((uint32_t)(key >> G.own_shift), __float_as_uint(L.run[key]));
+    const size_t at = ((size_t)owner * G.n_blocks + block) * kHandoffRecs + slot;
+    uint32_t tag = (uint32_t)(key >> G.own_shift);
+    if (slot == 0) {
+      const int c = L.handed[owner];  // final: every wave has had its turn
+      tag |= (uint32_t)(c > kSlotCap ? kSlotOverflow : c) << 8;
+    }
+    handoff[at] = make_uint2(tag, __float_as_uint(L.run[key]));
   }
-  if (tid < n_own) {
-    const int c = L.handed[tid];
-    handoff[((size_t)tid * G.n_blocks + block) * kHandoffRecs] =
-        make_uint2((uint32_t)(c > kSlotCap ? kSlotOverflow : c), 0u);
-  }
+  if (tid < n_own && L.handed[tid] == 0)
+    handoff[((size_t)tid * G.n_blocks + block) * kHandoffRecs] = make_uint2(0u, 0u);
 }
 
 // Pass 1 over (key, delta) arrays already in memory.
@@ -129,6 +152,7 @@ __global__ __launch_bounds__(kBlockSamples) void k_reduce_blocks(const ReduceGeo
                                                                  uint2* __restrict__ handoff) {
   extern __shared__ unsigned char lds_raw[];
   ReduceLds& L = *reinterpret_cast<ReduceLds*>(lds_raw);
+  reduce_block_clear(L, G);
   const int i = blockIdx.x * kBlockSamples + threadIdx.x;
   const int k = i < n ? key[i] : -1;
   const bool valid = k >= 0;
@@ -167,14 +191,13 @@ __global__ __launch_bounds__(256) void k_reduce_owners(const ReduceGeom G, float
     float4* my_row = reinterpret_cast<float4*>(tile + tid * kOwnKeys);
 #pragma unroll
     for (int i = 0; i < kOwnKeys / 4; ++i) my_row[i] = make_float4(0.0f, 0.0f, 0.0f, 0.0f);
-    const int c = (int)cell[0].x;
+    const int c = (int)((cell[0].x >> 8) & 0xFFu);
     if (c != kSlotOverflow) {
       float* row = tile + tid * kOwnKeys;
-      if (c > 0) row[cell[0].z] = __uint_as_float(cell[0].w);
 #pragma unroll
-      for (int i = 1; i < kHandoffRecs / 2; ++i) {
-        if (c > 2 * i - 1) row[cell[i].x] = __uint_as_float(cell[i].y);
-        if (c > 2 * i) row[cell[i].z] = __uint_as_float(cell[i].w);
+      for (int i = 0; i < kHandoffRecs / 2; ++i) {
+        if (c > 2 * i) row[cell[i].x & 0xFFu] = __uint_as_float(cell[i].y);
+        if (c > 2 * i + 1) row[cell[i].z & 0xFFu] = __uint_as_float(cell[i].w);
       }
     } else {
       // more distinct keys than slots: redo the block's part from its samples, in order
