@@ -49,9 +49,16 @@ __device__ __forceinline__ void action_delta(int a, int A, int& dx, int& dy) {
 // One move (src/kernels.cu:13-66 on cell classes; goal_mode 1 gives
 // src/environment.cu:17-48).  `cls(cell)` returns the class of a cell of this
 // env's map, `cr` its per-cell rewards (may be null when unused).
+// The reward is a class constant or ONE element of `cr`, at an index that is
+// known as soon as the class of the target cell is: a single load that is in
+// flight together with the table row of the new cell.
+struct ClassRewards {
+  float step, goal, trap;
+};
 template <class ClassOf>
-__device__ __forceinline__ void step_rule(const Rules& R, const ClassOf& cls, const float* __restrict__ cr,
-                                          int& x, int& y, int a, float& reward, bool& hit) {
+__device__ __forceinline__ void step_rule(const Rules& R, const ClassRewards by, const ClassOf& cls,
+                                          const float* __restrict__ cr, int& x, int& y, int a,
+                                          float& reward, bool& hit) {
   int dx, dy;
   action_delta(a, R.A, dx, dy);
   const int nx = x + dx, ny = y + dy;
@@ -59,29 +66,22 @@ __device__ __forceinline__ void step_rule(const Rules& R, const ClassOf& cls, co
   const int tgt = ny * R.W + nx;
   const int k = in ? cls(tgt) : kFree;
   const bool moved = in && k < kTrap;
-  if (moved) {
-    x = nx;
-    y = ny;
-  }
+  x = moved ? nx : x;
+  y = moved ? ny : y;
   const int s2 = y * R.W + x;
+  const bool trap = in && k == kTrap;
+  // goal test: on the target cell, or (goal_mode 1) on the cell the env ends up on,
+  // where it fires again while the env bumps into something next to the goal
+  hit = R.goal_mode == 0 ? (in && k == kGoal) : (cls(s2) == kGoal);
+  // goal beats trap; the goal pays on the goal cell (= s2 in both modes: a goal
+  // target is moved onto), the trap on the target cell, anything else on s2
   const bool cells = (R.reward_flags & 1) != 0;
-  float r = (cells && (R.reward_flags & 2)) ? cr[s2] : R.step_reward;
-  hit = false;
-  if (R.goal_mode == 0) {
-    if (in && k == kGoal) {
-      r = cells ? cr[tgt] : R.goal_reward;
-      hit = true;
-    } else if (in && k == kTrap) {
-      r = cells ? cr[tgt] : R.trap_reward;
-    }
-  } else {
-    if (in && k == kTrap) r = cells ? cr[tgt] : R.trap_reward;
-    if (cls(s2) == kGoal) {
-      r = cells ? cr[s2] : R.goal_reward;
-      hit = true;
-    }
-  }
-  reward = r;
+  const bool base_cells = cells && (R.reward_flags & 2) != 0;
+  const float by_class = hit ? by.goal : trap ? by.trap : by.step;
+  const bool from_cell = cells && (hit || trap || base_cells);
+  float by_cell = 0.0f;
+  if (cells) by_cell = cr[(trap && !hit) ? tgt : s2];  // uniform branch, index always inside the map
+  reward = from_cell ? by_cell : by_class;
 }
 
 // Move codes: what each action does from one cell, 2 bits per action -

@@ -161,14 +161,15 @@ __device__ __forceinline__ LdsMap<F> lds_map(F f) { return LdsMap<F>{f}; }
 // (cls.arrive(x, y) is called whenever the env lands on a cell), `cr` its
 // per-cell rewards (or null), `tab` its table.
 template <int A, class Table, class ClassOf>
-__device__ __forceinline__ void run_env_steps(const Rules& R_in, const Ptrs& P, const int env,
+__device__ __forceinline__ void run_env_steps(const Rules& R, const Ptrs& P, const int env,
                                               const uint64_t t0, const int n_steps, ClassOf& cls,
                                               const float* __restrict__ cr, const Table tab) {
   // The class rewards as plain register values.  As loads from the kernel's
   // argument block, "cell reward or class reward" is turned into one load through
   // a selected pointer, which needs the class rewards copied to scratch memory.
-  Rules R = R_in;
-  asm volatile("" : "+s"(R.step_reward), "+s"(R.goal_reward), "+s"(R.trap_reward));
+  float r_step = R.step_reward, r_goal = R.goal_reward, r_trap = R.trap_reward;
+  asm volatile("" : "+v"(r_step), "+v"(r_goal), "+v"(r_trap));
+  const ClassRewards by{r_step, r_goal, r_trap};
   const int start = P.start[env];
   const int sx = start % R.W, sy = start / R.W;
   int s = P.s[env];
@@ -206,33 +207,34 @@ __device__ __forceinline__ void run_env_steps(const Rules& R_in, const Ptrs& P, 
 
     const int s0 = s;
     bool hit;
-    step_rule(R, cls, cr, x, y, a, reward, hit);
+    step_rule(R, by, cls, cr, x, y, a, reward, hit);
     const int s2 = y * R.W + x;
     done = hit || (!R.auto_reset && done);
 
-    // Q row of the new cell; when the env did not move it is the row in registers.
-    // An env whose episode ends with this step also needs the row and the
-    // neighbourhood of its start cell: known now, so everything is requested in
-    // one go and a step has one memory round trip
-    Row<A> row2 = row;
-    const bool ends = R.auto_reset && (done || (R.episode_len > 0 && ep_step + 1 >= R.episode_len));
-    if (s2 != s0) row2 = tab.load(s2);
-    Row<A> row_start{};
-    if (ends) {
-      row_start = tab.load(start);
-      cls.arrive(sx, sy);
-    } else if (s2 != s0) {
-      cls.arrive(x, y);
-    }
+    // Everything the rest of this step and the start of the next one read from
+    // memory is asked for here, in one go: the row of the cell the move ends on
+    // (for the TD target), the row and the map neighbourhood of the cell the env
+    // acts from next - the same cell unless the episode ends with this step and
+    // the env restarts - and, inside step_rule, the reward.  One round trip per
+    // step, no branch around a load.  An env that stays where it is reads its own
+    // row again (the pre-update values: the write below comes later).
+    ep_step += 1;
+    const bool ends = R.auto_reset && (done || (R.episode_len > 0 && ep_step >= R.episode_len));
+    s = ends ? start : s2;
+    x = ends ? sx : x;
+    y = ends ? sy : y;
+    const Row<A> row2 = tab.load(s2);
+    const Row<A> row_next = tab.load(s);
+    cls.arrive(x, y);
     // the next step's draws depend on nothing: the Philox rounds run while the
     // loads are in flight
     if ((t & 1) == 1) blk = explore_block(R.seed, (uint32_t)env, (t + 1) >> 1);
-    row_opaque(row_start);
     const float m = row_max(row2, done, R.max_mode);
     const float qn = td_value(row_get(row, a), reward, m, R.lr, R.gamma);
     tab.store(s0, a, qn);
+    // the value just written, patched in from registers
+    row = row_set(row_next, s == s0 ? a : -1, qn);
 
-    ep_step += 1;
     action = a;
     ret = ret + reward;
     if (env < P.trace_n && P.trace_cursor + k < P.trace_cap) {
@@ -243,11 +245,6 @@ __device__ __forceinline__ void run_env_steps(const Rules& R_in, const Ptrs& P, 
       P.tr_d[o] = done ? 1 : 0;
     }
     if (ends && track) record_episode(P, env, ret, ep_step);
-    // the cell to act from next, with the value just written patched in from registers
-    s = ends ? start : s2;
-    row = row_set(ends ? row_start : row2, s == s0 ? a : -1, qn);
-    x = ends ? sx : x;
-    y = ends ? sy : y;
     ret = ends ? 0.0f : ret;
     ep_step = ends ? 0 : ep_step;
     episode += ends ? 1 : 0;
@@ -669,7 +666,7 @@ __global__ __launch_bounds__(256) void k_step(const Rules R, const Ptrs P, const
   const int a = act[env];
   float reward;
   bool hit;
-  step_rule(R, cls, cr, x, y, a, reward, hit);
+  step_rule(R, ClassRewards{R.step_reward, R.goal_reward, R.trap_reward}, cls, cr, x, y, a, reward, hit);
   const int s2 = y * R.W + x;
   const bool done = hit || (!R.auto_reset && P.done[env] != 0);
   int ep_step = P.ep_step[env] + 1;
@@ -828,7 +825,7 @@ __global__ __launch_bounds__(256) void k_shared_act(const Rules R, const Ptrs P,
     const int a = (d.u < eps) ? d.a : row_argmax(row);
     float reward;
     bool hit;
-    step_rule(R, cls, cr, x, y, a, reward, hit);
+    step_rule(R, ClassRewards{R.step_reward, R.goal_reward, R.trap_reward}, cls, cr, x, y, a, reward, hit);
     const int s2 = y * R.W + x;
     const bool done = hit || (!R.auto_reset && P.done[env] != 0);
     float m = row_max(row, false, 0);  // the env stayed where it was
