@@ -125,6 +125,21 @@ __device__ __forceinline__ uint32_t moves_of_cell(WordOf word_of, int W, int H, 
 template <int A>
 __device__ __forceinline__ constexpr int move_cells_per_word() { return 16 / A; }
 
+// 16-byte loads / stores marked non-temporal: data that streams through once
+typedef float crl_f4 __attribute__((ext_vector_type(4)));
+__device__ __forceinline__ float4 stream_load4(const float4* p) {
+  const crl_f4 v = __builtin_nontemporal_load(reinterpret_cast<const crl_f4*>(p));
+  return make_float4(v.x, v.y, v.z, v.w);
+}
+__device__ __forceinline__ void stream_store4(const float4 v, float4* p) {
+  crl_f4 t;
+  t.x = v.x;
+  t.y = v.y;
+  t.z = v.z;
+  t.w = v.w;
+  __builtin_nontemporal_store(t, reinterpret_cast<crl_f4*>(p));
+}
+
 // One table row in registers.  Named scalars passed BY VALUE: an element picked
 // by a run-time action index must compile to a chain of selects.  Through a
 // reference the optimiser folds "select of two loads" into one indexed load

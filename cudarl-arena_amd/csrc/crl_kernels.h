@@ -477,7 +477,7 @@ __device__ __forceinline__ void stage_words(const uint32_t* __restrict__ src, co
                                             const int lane) {
   for (int i = lane; i < count * wpe; i += 64) {
     const int e = i / wpe, w = i - e * wpe;
-    dst[w * stride + e] = src[i];
+    dst[w * stride + e] = __builtin_nontemporal_load(src + i);  // read once per launch
   }
 }
 
@@ -541,6 +541,9 @@ __global__ __launch_bounds__(LDSW ? 320 : 256) void k_fused_tickets(const Rules 
       const float4* g4 = reinterpret_cast<const float4*>(P.Q + (size_t)env0 * table);
       const int t4 = (int)(table / 4);
       const int total4 = n_here * t4;
+      // streamed once in and once out: marked non-temporal so that they do not
+      // push the table waves' rows out of the L2
+      auto ld = [&](int i) -> float4 { return stream_load4(g4 + i); };
       auto put = [&](int i, const float4 v) {
         const int e = i / t4, o = i - e * t4;
         reinterpret_cast<float4*>(tabs + e * tab_stride)[o] = v;
@@ -548,8 +551,8 @@ __global__ __launch_bounds__(LDSW ? 320 : 256) void k_fused_tickets(const Rules 
       int i0 = 0;
       for (; i0 + 64 * 8 <= total4; i0 += 64 * 8) {  // eight loads in flight per lane
         const int i = i0 + lane;
-        const float4 v0 = g4[i], v1 = g4[i + 64], v2 = g4[i + 128], v3 = g4[i + 192];
-        const float4 v4 = g4[i + 256], v5 = g4[i + 320], v6 = g4[i + 384], v7 = g4[i + 448];
+        const float4 v0 = ld(i), v1 = ld(i + 64), v2 = ld(i + 128), v3 = ld(i + 192);
+        const float4 v4 = ld(i + 256), v5 = ld(i + 320), v6 = ld(i + 384), v7 = ld(i + 448);
         put(i, v0);
         put(i + 64, v1);
         put(i + 128, v2);
@@ -559,7 +562,7 @@ __global__ __launch_bounds__(LDSW ? 320 : 256) void k_fused_tickets(const Rules 
         put(i + 384, v6);
         put(i + 448, v7);
       }
-      for (int i = i0 + lane; i < total4; i += 64) put(i, g4[i]);
+      for (int i = i0 + lane; i < total4; i += 64) put(i, ld(i));
       __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
       __builtin_amdgcn_wave_barrier();
       if (FAST) {
@@ -584,12 +587,12 @@ __global__ __launch_bounds__(LDSW ? 320 : 256) void k_fused_tickets(const Rules 
       for (; j0 + 64 * 4 <= total4; j0 += 64 * 4) {
         const int i = j0 + lane;
         const float4 v0 = get(i), v1 = get(i + 64), v2 = get(i + 128), v3 = get(i + 192);
-        o4[i] = v0;
-        o4[i + 64] = v1;
-        o4[i + 128] = v2;
-        o4[i + 192] = v3;
+        stream_store4(v0, o4 + i);
+        stream_store4(v1, o4 + i + 64);
+        stream_store4(v2, o4 + i + 128);
+        stream_store4(v3, o4 + i + 192);
       }
-      for (int i = j0 + lane; i < total4; i += 64) o4[i] = get(i);
+      for (int i = j0 + lane; i < total4; i += 64) stream_store4(get(i), o4 + i);
     }
   }
 }
