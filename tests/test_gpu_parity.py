@@ -511,6 +511,31 @@ def test_full_size_config4(gpu, oracle):
     assert (st["ep_step"] < 128).all() and st["episode"].min() >= steps // 128
 
 
+@pytest.mark.parametrize("fixture", ["baseline", "reference"])
+def test_full_size_config1(gpu, oracle, fixture):
+    """Config 1, whole program: one 10x10 grid without walls, 1000 episodes of at
+    most 500 steps, eps 1.0 decaying x0.995.  Two fixtures: the benchmark's wording
+    (start (0,0), goal (9,9), decay per episode) and the reference's default world
+    (start (5,5), goal (9,0): src/environment.cu:9-10,146; decay per update:
+    src/train.py:140-141).  Every step of every episode is compared."""
+    W = H = 10
+    E, T = 1000, 500
+    cls = np.zeros(W * H, np.uint8)
+    if fixture == "baseline":
+        start, goal = [0], 9 * W + 9
+        sched = dict(eps_mode=gpu.EPS_EPISODE_MULT, eps_span=E + 1)
+    else:
+        start, goal = [(H // 2) * W + W // 2], W - 1
+        sched = dict(eps_mode=gpu.EPS_STEP_MULT, eps_span=E * T + 1)
+    cls[goal] = gpu.CELL_GOAL
+    cfg = gpu.make_config(1, W, H, map_mode=gpu.MAP_SHARED, episode_len=T, lr=0.1, gamma=0.99, eps0=1.0,
+                          eps_decay=0.995, max_episodes=E, seed=0, **sched)
+    tr, q = run_both(gpu, oracle, cfg, cls, start, E * T)
+    ends = int(tr["done"].sum())
+    assert ends > E // 2  # most episodes reach the goal once the table has learnt the way
+    assert float(q.max()) > 0.9
+
+
 def test_full_size_config2(gpu, oracle):
     """4096 envs, 32x32, 256-step episodes, all 10,000 steps: final tables and
     state bit-exact against the oracle."""
