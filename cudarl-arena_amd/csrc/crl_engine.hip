@@ -207,7 +207,7 @@ struct FusedPlan {
   size_t lds;
   const char* name;
   bool tickets;    // per-env maps in LDS: waves draw env ranges from a ticket counter
-  bool hybrid;     // ... with a fifth wave per workgroup that steps envs whose tables it holds in LDS
+  bool hybrid;     // ... whose last wave per workgroup steps envs whose tables it holds in LDS
   bool fast;       // the folded loop for the common configuration
   bool moves;      // ... whose table waves read pre-built move codes from LDS
   int tab_stride;  // floats between two tables in LDS

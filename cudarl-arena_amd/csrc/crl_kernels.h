@@ -94,7 +94,9 @@ __device__ __forceinline__ Draw pick_draw(const Philox4 blk, uint64_t t, int A) 
 // Fused select -> step -> update, per-env tables, one lane per env, n_steps per
 // launch.  The env's position, episode counters and the Q row of the cell it
 // stands on live in registers for the whole launch: per step the only table
-// traffic is one row read (the new cell) and one 4-byte write.
+// traffic is the row of the new cell (asked for twice when the episode goes on:
+// as the TD target's row and as the next row to act from - one cache line) and
+// one 4-byte write.
 // ---------------------------------------------------------------------------
 
 // where an env's table lives while it is being stepped
@@ -158,7 +160,7 @@ template <class F>
 __device__ __forceinline__ LdsMap<F> lds_map(F f) { return LdsMap<F>{f}; }
 
 // n_steps of one env.  `cls(cell)` gives the class of a cell of the env's map
-// (cls.arrive(x, y) is called whenever the env lands on a cell), `cr` its
+// (cls.arrive(x, y) is called with the cell the env acts from next), `cr` its
 // per-cell rewards (or null), `tab` its table.
 template <int A, class Table, class ClassOf>
 __device__ __forceinline__ void run_env_steps(const Rules& R, const Ptrs& P, const int env,

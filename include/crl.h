@@ -127,7 +127,7 @@ int crl_sync(crl_engine* e);
 int crl_set_resident_envs(crl_engine* e, int32_t n_envs);
 /* Tuning (no reference counterpart): kernel of crl_run_fused for per-env tables.
  * 0 = automatic, 1 = plain (every wave steps envs against tables in HBM),
- * 2 = hybrid (a fifth wave per workgroup steps envs whose whole tables it holds
+ * 2 = hybrid (the last wave of each workgroup steps envs whose whole tables it holds
  * in LDS; used only when 32 tables fit).  Results do not depend on it. */
 int crl_set_fused_variant(crl_engine* e, int32_t variant);
 /* How the last hybrid crl_run_fused split the envs between its two kinds of

@@ -85,7 +85,7 @@ def test_fused_chunked_equals_one_launch(gpu, oracle):
 
 def test_fused_result_independent_of_resident_envs(gpu, oracle):
     """Few envs in flight (blocks loop over chunks, re-staging maps) == all at once,
-    for the plain kernel and for the hybrid one (a fifth wave per workgroup steps
+    for the plain kernel and for the hybrid one (the last wave of each workgroup steps
     envs whose tables it holds in LDS; N is not a multiple of the 32-env ticket)."""
     N, W, H, T = 3001, 16, 16, 150
     cls, start = gpu.gen_maps_bernoulli(31, N, N, W, H, 0.1, 0.02)
