@@ -194,8 +194,8 @@ namespace {
 
 constexpr int kLdsMapLimitBytes = 64 * 1024;
 // Table bytes to keep in flight at once: three quarters of the MI355X Infinity
-// Cache (256 MB).  Measured on 4 KB tables: 128 MB in flight 4.1e10 env-steps/s,
-// 192 MB 4.9e10, 256 MB 4.5e10, 384 MB 3.7e10.
+// Cache (256 MB).  Measured on 4 KB tables (table waves alone): 128 MB in flight 5.9e10 env-steps/s,
+// 192 MB 6.3e10, 256 MB 5.2e10, 384 MB 3.9e10.
 constexpr size_t kTableBytesInFlight = (size_t)192 << 20;
 constexpr int kComputeUnits = 256;
 constexpr long kMinEnvsInFlight = kComputeUnits * 3L * 64;  // three waves per compute unit
