@@ -91,7 +91,8 @@ def test_fused_result_independent_of_resident_envs(gpu, oracle):
     cls, start = gpu.gen_maps_bernoulli(31, N, N, W, H, 0.1, 0.02)
     cfg = gpu.make_config(N, W, H, episode_len=40, eps0=0.2, gamma=0.95, seed=17)
     outs = []
-    for resident, variant in ((0, 1), (64, 1), (640, 1), (1000, 1), (0, 2), (256, 2), (1024, 2)):
+    for resident, variant in ((0, 1), (64, 1), (640, 1), (1000, 1), (0, 2), (256, 2), (1024, 2), (1500, 2), (2200, 2),
+                              (3000, 2)):
         with gpu.Engine(cfg, 0) as eng:
             eng.set_maps(cls, start)
             eng.set_resident_envs(resident)
