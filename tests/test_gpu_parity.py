@@ -144,6 +144,31 @@ def test_fused_fast_loop_matches_oracle(gpu, oracle, variant, N, W, H, T, steps,
     assert st["episode"].max() >= 1
 
 
+@pytest.mark.parametrize("variant", [1, 2])
+def test_fused_fast_loop_short_launches_no_time_limit(gpu, oracle, variant):
+    """The folded loop in launches of 0, 1, 2 and 3 steps (tables staged in and out
+    of LDS around a single step; odd and even first steps) and without a time limit
+    (episodes end on the goal only)."""
+    N, W, H = 2300, 12, 12
+    cls, start = gpu.gen_maps_bernoulli(53, N, N, W, H, 0.1, 0.02)
+    cfg = gpu.make_config(N, W, H, episode_len=0, eps0=0.25, gamma=0.9, seed=31)
+    chunks = [1, 0, 1, 2, 3, 1, 40, 1]
+    with gpu.Engine(cfg, 0) as eng:
+        eng.set_maps(cls, start)
+        eng.set_fused_variant(variant)
+        assert "fast" in eng.fused_kernel_info()["name"]
+        for c in chunks:
+            eng.run_fused(c)
+        q, st = eng.q_get(0, N), eng.get_state()
+        assert eng.step_count == sum(chunks)
+    Q = np.zeros((N, W * H, 4), np.float32)
+    ost = oracle.new_state(cfg, start)
+    oracle.run(cfg, cls, None, start, Q, ost, 0, sum(chunks))
+    for k in ("s", "ep_step", "episode", "reward", "done", "action"):
+        assert np.array_equal(st[k], ost[k]), k
+    assert_q_close(q.reshape(Q.shape), Q)
+
+
 @pytest.mark.parametrize("variant,resident", [(1, 0), (1, 192), (2, 0)])
 @pytest.mark.parametrize("N,W,H,A", [(2500, 16, 16, 8), (300, 9, 6, 8), (2100, 7, 5, 4), (130, 33, 31, 4)])
 def test_fused_fast_loop_move_codes(gpu, oracle, variant, resident, N, W, H, A):
