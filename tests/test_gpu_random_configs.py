@@ -1,0 +1,109 @@
+"""GPU parity on randomly drawn configurations: every switch of the configuration
+(actions, grid shape, table and map sharing, reward source, goal rule, restart,
+time limit, epsilon schedule, TD max, episode budget, trace, kernel variant, envs
+in flight, launch splits) in combinations no hand-written case lists.  Final
+state and tables - and the whole trajectory when traced - must be the oracle's,
+bit for bit.  Seeds are fixed: a failure names its case."""
+import numpy as np
+import pytest
+
+pytestmark = pytest.mark.gpu
+
+STATE = ("s", "ep_step", "episode", "reward", "done", "action")
+
+
+def same(gpu_q, gpu_state, Q, ost):
+    return (np.array_equal(gpu_q.reshape(Q.shape), Q, equal_nan=True) and
+            all(np.array_equal(gpu_state[k], ost[k]) for k in STATE))
+
+
+@pytest.mark.parametrize("seed", [1, 2, 3])
+def test_random_configs_folded_loop(gpu, oracle, seed):
+    """The common configuration (fixed epsilon, class rewards, goal on the target
+    cell, restart) on per-env tables: the folded loop of both kinds of workers."""
+    rng = np.random.default_rng(seed)
+    for case in range(40):
+        A = int(rng.choice([4, 8]))
+        small = rng.random() < 0.5  # small grids: 32 whole tables fit LDS
+        W, H = (int(rng.integers(2, 17 if small else 40)) for _ in range(2))
+        N = int(rng.choice([1, 31, 33, 64, 65, 500, 2049, 4100, 9000]))
+        T = int(rng.choice([0, 1, 2, 7, 50, 300]))
+        steps, t0 = int(rng.integers(1, 200)), int(rng.integers(0, 5))
+        eps = float(rng.choice([0.0, 0.05, 0.3, 1.0]))
+        variant, resident = int(rng.choice([0, 1, 2])), int(rng.choice([0, 64, 200, 1000, 5000]))
+        p_wall, p_trap = float(rng.choice([0.0, 0.1, 0.3])), float(rng.choice([0.0, 0.05]))
+        map_seed = int(rng.integers(0, 1 << 30))
+        cls, start = gpu.gen_maps_bernoulli(map_seed, N, N, W, H, p_wall, p_trap)
+        cfg = gpu.make_config(N, W, H, n_actions=A, episode_len=T, eps0=eps, gamma=0.93, lr=0.2, seed=map_seed,
+                              trap_reward=-0.7)
+        with gpu.Engine(cfg, 0) as eng:
+            eng.set_maps(cls, start)
+            eng.set_fused_variant(variant)
+            eng.set_resident_envs(resident)
+            eng.step_count = t0
+            name = eng.fused_kernel_info()["name"]
+            third = steps // 3
+            for c in (third, steps - 2 * third, third):
+                eng.run_fused(c)
+            q, st = eng.q_get(0, N), eng.get_state()
+        Q = np.zeros((N, W * H, A), np.float32)
+        ost = oracle.new_state(cfg, start)
+        oracle.run(cfg, cls, None, start, Q, ost, t0, steps)
+        assert "fast" in name
+        assert same(q, st, Q, ost), (seed, case, name, A, W, H, N, T, steps, t0, eps, variant, resident)
+
+
+@pytest.mark.parametrize("seed", [1, 7])
+def test_random_configs_general(gpu, oracle, seed):
+    """Everything else: shared tables and maps, maps too large for LDS, per-cell
+    rewards, goal test on the resulting cell, sticky done, epsilon schedules, the
+    zero-floored max, episode budgets, traces."""
+    rng = np.random.default_rng(seed)
+    for case in range(60):
+        A = int(rng.choice([4, 8]))
+        big = rng.random() < 0.25  # more than 4096 cells: the map stays in global memory
+        W, H = (int(rng.integers(65, 90)) if big else int(rng.integers(2, 30)) for _ in range(2))
+        shared_table = rng.random() < 0.35
+        shared_map = shared_table or rng.random() < 0.3
+        N = int(rng.choice([5, 70, 300] if big else [1, 33, 257, 700, 3000]))
+        T = int(rng.choice([0, 1, 3, 20, 100]))
+        steps = int(rng.integers(1, 90 if shared_table else 200))
+        eps_mode, span = int(rng.choice([0, 1, 2, 3])), int(rng.integers(1, 50))
+        flags = int(rng.choice([0, gpu.REWARD_CELLS, gpu.REWARD_CELLS | gpu.REWARD_BASE_CELLS]))
+        goal_mode, max_mode = int(rng.choice([0, 1])), int(rng.choice([0, 1]))
+        auto_reset = int(rng.choice([0, 1, 1]))
+        max_episodes = int(rng.choice([0, 0, 2])) if auto_reset else 0
+        map_seed = int(rng.integers(0, 1 << 30))
+        n_maps = 1 if shared_map else N
+        if flags:
+            cls, start, cr = gpu.gen_maps_noise(map_seed, n_maps, W, H, 8, 0.2, 0.3, 5.0)
+            start = np.resize(start, N).astype(np.int32)
+        else:
+            cls, start = gpu.gen_maps_bernoulli(map_seed, n_maps, N, W, H, 0.15, 0.05)
+            cr = None
+        cfg = gpu.make_config(N, W, H, n_actions=A,
+                              table_mode=gpu.TABLE_SHARED if shared_table else gpu.TABLE_PER_ENV,
+                              map_mode=gpu.MAP_SHARED if shared_map else gpu.MAP_PER_ENV, max_mode=max_mode,
+                              goal_mode=goal_mode, auto_reset=auto_reset, episode_len=T,
+                              lr=0.002 if shared_table else 0.2, gamma=0.9, reward_flags=flags, eps_mode=eps_mode,
+                              eps0=0.6, eps_decay=0.97, eps_end=0.05, eps_span=span, seed=map_seed,
+                              max_episodes=max_episodes, trap_reward=-0.5)
+        n_tables = 1 if shared_table else N
+        trace_n = N if rng.random() < 0.5 else 0
+        with gpu.Engine(cfg, 0) as eng:
+            eng.set_maps(cls, start, cr)
+            if trace_n:
+                eng.set_trace(trace_n, steps)
+            name = eng.fused_kernel_info()["name"]
+            eng.run_fused(steps // 2)
+            eng.run_fused(steps - steps // 2)
+            tr = eng.get_trace(steps) if trace_n else None
+            q, st = eng.q_get(0, n_tables), eng.get_state()
+        Q = np.zeros((n_tables, W * H, A), np.float32)
+        ost = oracle.new_state(cfg, start)
+        want = oracle.run(cfg, cls, cr, start, Q, ost, 0, steps, trace_n=trace_n)
+        what = (seed, case, name, A, W, H, N, T, steps, eps_mode, flags, goal_mode, auto_reset, max_mode,
+                max_episodes, shared_table, shared_map, trace_n)
+        assert same(q, st, Q, ost), what
+        if trace_n:
+            assert all(np.array_equal(tr[k], want[k]) for k in ("s_next", "action", "reward", "done")), what
