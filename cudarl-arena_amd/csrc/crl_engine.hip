@@ -221,9 +221,9 @@ FusedPlan plan_fused(const crl_engine* e) {
   // small batches spread over more compute units with one-wave blocks
   p.block = e->N >= 256 * 512 ? 256 : 64;
   if (e->cfg.map_mode == CRL_MAP_SHARED) {
-    if ((size_t)e->map_words * 4 <= (size_t)kLdsMapLimitBytes) {
+    if ((size_t)e->mv_words * 4 <= (size_t)kLdsMapLimitBytes) {
       p.map_kind = 1;
-      p.lds = (size_t)e->map_words * 4;
+      p.lds = (size_t)e->mv_words * 4;  // the shared map's move codes
     } else {
       p.map_kind = 2;
     }
@@ -570,8 +570,8 @@ int crl_create(const crl_config* cfg, int device, crl_engine** out) {
   acc(e->done.alloc(N));
   acc(e->action.alloc(N));
   acc(e->map.alloc((size_t)e->n_maps * e->map_words));
-  // move codes for the folded fused loop: per-env maps that the ticket kernel stages in LDS
-  if (cfg->map_mode != CRL_MAP_SHARED && (size_t)e->map_words * 4 * 64 <= (size_t)kLdsMapLimitBytes) {
+  // move codes of every map, for the fused loops
+  {
     const size_t cells_per_word = 16 / (size_t)e->A;
     e->mv_words = (int)((e->S + cells_per_word - 1) / cells_per_word);
     acc(e->moves.alloc((size_t)e->n_maps * e->mv_words));

@@ -124,83 +124,88 @@ struct LdsTable {  // staged into LDS for the whole launch
   __device__ __forceinline__ void store(int s, int a, float v) const { q[s * A + a] = v; }
 };
 
-// A map too large for LDS, read from global memory: the words that hold the
-// 3 x 3 cells around the env are fetched when it ARRIVES on a cell (together with
-// the table row of that cell), so that the class of the next target comes from
-// registers and a step has one memory round trip on its critical path, not two.
-struct NearMap {
-  const uint32_t* g;
+// Where the fused loops get the move codes of a cell from.
+// Pre-built codes staged in LDS, word-interleaved over the wave's lanes:
+template <int A>
+struct MovesLds {
+  const uint32_t* base;  // the lane's first word
+  int stride;            // words between two consecutive words of one env
+  __device__ __forceinline__ uint32_t at(int s, int, int) const {
+    constexpr unsigned kCells = (unsigned)move_cells_per_word<A>();
+    const unsigned c = (unsigned)s;  // cell indices are never negative: shifts, not signed division
+    return base[(c / kCells) * (unsigned)stride] >> ((c % kCells) * 2u * A);
+  }
+};
+// Derived from the class map in LDS when the codes of all lanes do not fit: one
+// map word per action, asked for while the table row is in flight.
+template <int A>
+struct MovesFromMap {
+  const uint32_t* base;  // the lane's first map word, words 64 apart
   int W, H;
-  uint32_t w0, w1, w2, w3, w4, w5;  // rows y-1, y, y+1: the words of x-1 and of x+1
-  int i0, i1, i2, i3, i4, i5;       // their word indices
-  __device__ __forceinline__ void arrive(int x, int y) {
-    const int xl = max(x - 1, 0), xr = min(x + 1, W - 1);
-    const int ya = max(y - 1, 0) * W, yb = y * W, yc = min(y + 1, H - 1) * W;
-    i0 = (ya + xl) >> 4; i1 = (ya + xr) >> 4;
-    i2 = (yb + xl) >> 4; i3 = (yb + xr) >> 4;
-    i4 = (yc + xl) >> 4; i5 = (yc + xr) >> 4;
-    w0 = g[i0]; w1 = g[i1]; w2 = g[i2]; w3 = g[i3]; w4 = g[i4]; w5 = g[i5];
-  }
-  // the words of the last arrive() have landed (a loop entered with loads still
-  // in flight waits for every outstanding memory operation on each iteration)
-  __device__ __forceinline__ void settle() {
-    asm volatile("" : "+v"(w0), "+v"(w1), "+v"(w2), "+v"(w3), "+v"(w4), "+v"(w5));
-  }
-  // class of a cell at most one step away from the cell of the last arrive()
-  __device__ __forceinline__ int operator()(int cell) const {
-    const int i = cell >> 4;
-    uint32_t w = w0;
-    w = (i == i1) ? w1 : w;
-    w = (i == i2) ? w2 : w;
-    w = (i == i3) ? w3 : w;
-    w = (i == i4) ? w4 : w;
-    w = (i == i5) ? w5 : w;
-    return cell_class_of(w, cell);
+  __device__ __forceinline__ uint32_t at(int s, int x, int y) const {
+    return moves_of_cell<A>([&](int word) -> uint32_t { return base[word * 64]; }, W, H, x, y, s);
   }
 };
 
-// a map in LDS needs no such preparation
-template <class F>
-struct LdsMap {
-  F word_of;  // cell -> packed word
-  __device__ __forceinline__ void arrive(int, int) {}
-  __device__ __forceinline__ void settle() {}
-  __device__ __forceinline__ int operator()(int cell) const { return cell_class_of(word_of(cell), cell); }
+// Read from global memory, for maps whose codes do not fit LDS: one load, in
+// flight together with the table row of the same cell.
+template <int A>
+struct MovesGlobal {
+  const uint32_t* base;  // the env's (or the shared) packed move codes
+  __device__ __forceinline__ uint32_t at(int s, int, int) const {
+    constexpr unsigned kCells = (unsigned)move_cells_per_word<A>();
+    const unsigned c = (unsigned)s;
+    return base[c / kCells] >> ((c % kCells) * 2u * A);
+  }
 };
-template <class F>
-__device__ __forceinline__ LdsMap<F> lds_map(F f) { return LdsMap<F>{f}; }
 
-// n_steps of one env.  `cls(cell)` gives the class of a cell of the env's map
-// (cls.arrive(x, y) is called with the cell the env acts from next), `cr` its
-// per-cell rewards (or null), `tab` its table.
-template <int A, class Table, class ClassOf>
+// n_steps of one env, any configuration.  `moves.at(cell, x, y)` gives the move
+// codes of a cell of the env's map, `own_map` is the env's packed class map in
+// global memory (read twice per launch, and only for the goal test on the
+// resulting cell), `cr` its per-cell rewards (or null), `tab` its table.
+// The step rule is step_rule()'s, restated on move codes: the class of the
+// target cell is two bits of the codes of the cell the env stands on.
+template <int A, class Table, class Moves>
 __device__ __forceinline__ void run_env_steps(const Rules& R, const Ptrs& P, const int env,
-                                              const uint64_t t0, const int n_steps, ClassOf& cls,
+                                              const uint64_t t0, const int n_steps, const Moves moves,
+                                              const uint32_t* __restrict__ own_map,
                                               const float* __restrict__ cr, const Table tab) {
   // The class rewards as plain register values.  As loads from the kernel's
   // argument block, "cell reward or class reward" is turned into one load through
   // a selected pointer, which needs the class rewards copied to scratch memory.
   float r_step = R.step_reward, r_goal = R.goal_reward, r_trap = R.trap_reward;
   asm volatile("" : "+v"(r_step), "+v"(r_goal), "+v"(r_trap));
-  const ClassRewards by{r_step, r_goal, r_trap};
-  const int start = P.start[env];
-  const int sx = start % R.W, sy = start / R.W;
+  const int W = R.W;
+  const bool cells = (R.reward_flags & 1) != 0;
+  const bool base_cells = cells && (R.reward_flags & 2) != 0;
+  const bool goal_on_result = R.goal_mode != 0;
+  int start = P.start[env];
+  const int sx = start % W, sy = start / W;
   int s = P.s[env];
-  int x = s % R.W, y = s / R.W;
+  int x = s % W, y = s / W;  // only followed when the move codes are derived from the map
   int ep_step = P.ep_step[env];
   int episode = P.episode[env];
   bool done = P.done[env] != 0;
   float reward = P.reward[env];  // rewritten unchanged if the env's episode budget is used up
   int action = P.action[env];
   Row<A> row = tab.load(s);
-  cls.arrive(x, y);
+  uint32_t mv = moves.at(s, x, y);
+  // goal test on the resulting cell: whether the env stands on a goal is carried
+  // along (a move onto a cell tells its class); the start cell's answer is fixed
+  int on_goal = 0, start_goal = 0;
+  if (goal_on_result) {
+    on_goal = cell_class_of(own_map[s >> 4], s) == kGoal;
+    start_goal = cell_class_of(own_map[start >> 4], start) == kGoal;
+  }
   Philox4 blk = explore_block(R.seed, (uint32_t)env, t0 >> 1);
   const bool track = P.ret_acc != nullptr;
   float ret = track ? P.ret_acc[env] : 0.0f;
-  // nothing loaded above is still in flight when the loop starts
+  // nothing loaded above is still in flight when the loop starts (a value still in
+  // flight at the loop's entry makes the loop wait for ALL outstanding memory
+  // operations on every iteration, the previous step's stores included)
   row_opaque(row);
-  cls.settle();
-  asm volatile("" : "+v"(ep_step), "+v"(episode), "+v"(reward), "+v"(action), "+v"(ret));
+  asm volatile("" : "+v"(ep_step), "+v"(episode), "+v"(reward), "+v"(action), "+v"(ret), "+v"(mv),
+               "+v"(start), "+v"(s), "+v"(on_goal), "+v"(start_goal));
 
   for (int k = 0; k < n_steps; ++k) {
     if (R.max_episodes > 0 && episode >= R.max_episodes) {
@@ -218,27 +223,43 @@ __device__ __forceinline__ void run_env_steps(const Rules& R, const Ptrs& P, con
     const float eps = eps_of(R, P.eps_tab, t, episode);
     const int a = (d.u < eps) ? d.a : row_argmax(row);
 
+    // the move (src/kernels.cu:13-66; goal on the resulting cell: src/environment.cu:43)
     const int s0 = s;
-    bool hit;
-    step_rule(R, by, cls, cr, x, y, a, reward, hit);
-    const int s2 = y * R.W + x;
+    const uint32_t code = (mv >> (2 * a)) & 3u;  // class of the target cell, WALL outside the grid
+    const bool moved = code < (uint32_t)kTrap;
+    const bool trap = code == (uint32_t)kTrap;
+    int dx, dy;
+    action_delta(a, A, dx, dy);
+    const int tgt = s0 + __mul24(dy, W) + dx;  // inside the map whenever it is used
+    const int s2 = moved ? tgt : s0;
+    dx = moved ? dx : 0;
+    dy = moved ? dy : 0;
+    const int on_goal2 = moved ? (int)(code == (uint32_t)kGoal) : on_goal;
+    const bool hit = goal_on_result ? on_goal2 != 0 : code == (uint32_t)kGoal;
+    // goal beats trap; the goal pays on the goal cell (= s2 under both rules), the
+    // trap on the target cell, anything else on s2: one load at one index
+    const float by_class = hit ? r_goal : trap ? r_trap : r_step;
+    float by_cell = 0.0f;
+    if (cells) by_cell = cr[(trap && !hit) ? tgt : s2];
+    reward = (cells && (hit || trap || base_cells)) ? by_cell : by_class;
     done = hit || (!R.auto_reset && done);
 
     // Everything the rest of this step and the start of the next one read from
-    // memory is asked for here, in one go: the row of the cell the move ends on
-    // (for the TD target), the row and the map neighbourhood of the cell the env
-    // acts from next - the same cell unless the episode ends with this step and
-    // the env restarts - and, inside step_rule, the reward.  One round trip per
-    // step, no branch around a load.  An env that stays where it is reads its own
-    // row again (the pre-update values: the write below comes later).
+    // memory is asked for here, in one go: the reward above, the row of the cell
+    // the move ends on (for the TD target), the row and the move codes of the cell
+    // the env acts from next - the same cell unless the episode ends with this
+    // step and the env restarts.  One round trip per step, no branch around a
+    // load.  An env that stays where it is reads its own row again (the pre-update
+    // values: the write below comes later).
     ep_step += 1;
     const bool ends = R.auto_reset && (done || (R.episode_len > 0 && ep_step >= R.episode_len));
     s = ends ? start : s2;
-    x = ends ? sx : x;
-    y = ends ? sy : y;
+    x = ends ? sx : x + dx;
+    y = ends ? sy : y + dy;
+    on_goal = ends ? start_goal : on_goal2;
     const Row<A> row2 = tab.load(s2);
     const Row<A> row_next = tab.load(s);
-    cls.arrive(x, y);
+    mv = moves.at(s, x, y);
     // the next step's draws depend on nothing: the Philox rounds run while the
     // loads are in flight
     if ((t & 1) == 1) blk = explore_block(R.seed, (uint32_t)env, (t + 1) >> 1);
@@ -271,29 +292,6 @@ __device__ __forceinline__ void run_env_steps(const Rules& R, const Ptrs& P, con
   P.done[env] = done ? 1 : 0;
   P.action[env] = (uint8_t)action;
 }
-
-// Where the folded loop gets the move codes of a cell from.
-// Pre-built codes staged in LDS, word-interleaved over the wave's lanes:
-template <int A>
-struct MovesLds {
-  const uint32_t* base;  // the lane's first word
-  int stride;            // words between two consecutive words of one env
-  __device__ __forceinline__ uint32_t at(int s, int, int) const {
-    constexpr unsigned kCells = (unsigned)move_cells_per_word<A>();
-    const unsigned c = (unsigned)s;  // cell indices are never negative: shifts, not signed division
-    return base[(c / kCells) * (unsigned)stride] >> ((c % kCells) * 2u * A);
-  }
-};
-// Derived from the class map in LDS when the codes of all lanes do not fit: one
-// map word per action, asked for while the table row is in flight.
-template <int A>
-struct MovesFromMap {
-  const uint32_t* base;  // the lane's first map word, words 64 apart
-  int W, H;
-  __device__ __forceinline__ uint32_t at(int s, int x, int y) const {
-    return moves_of_cell<A>([&](int word) -> uint32_t { return base[word * 64]; }, W, H, x, y, s);
-  }
-};
 
 // The same loop for the common configuration, with everything that is fixed
 // there folded away: fixed epsilon, class rewards (no per-cell array), goal test
@@ -430,9 +428,10 @@ __device__ __forceinline__ void run_env_fast(const Rules& R, const Ptrs& P, cons
   P.action[env] = (uint8_t)action;
 }
 
-// Per-env tables whose maps are shared (MAP = 1: the one map staged in LDS) or
-// too large for LDS (MAP = 2: read from global memory).  A block takes chunks
-// blockIdx, blockIdx + gridDim, ... and runs each for all n_steps.
+// Per-env tables whose maps are shared (MAP = 1: the one map's move codes staged
+// in LDS) or too large for LDS (MAP = 2: move codes read from global memory, one
+// load per step).  A block takes chunks blockIdx, blockIdx + gridDim, ... and runs
+// each for all n_steps.
 template <int A, int MAP>
 __global__ __launch_bounds__(256) void k_fused_per_env(const Rules R, const Ptrs P,
                                                         const uint64_t t0, const int n_steps) {
@@ -442,7 +441,7 @@ __global__ __launch_bounds__(256) void k_fused_per_env(const Rules R, const Ptrs
   const int n_chunks = (P.N + bdim - 1) / bdim;
 
   if (MAP == 1) {
-    for (int i = tid; i < P.map_words; i += bdim) lds[i] = P.map[i];
+    for (int i = tid; i < P.mv_words; i += bdim) lds[i] = P.moves[i];
     __syncthreads();
   }
   for (int chunk = blockIdx.x; chunk < n_chunks; chunk += gridDim.x) {
@@ -450,16 +449,13 @@ __global__ __launch_bounds__(256) void k_fused_per_env(const Rules R, const Ptrs
     if (env >= P.N) continue;
     const float* cr =
         P.cell_reward ? P.cell_reward + (P.map_shared ? 0 : (size_t)env * P.S) : nullptr;
+    const uint32_t* own_map = P.map + (P.map_shared ? 0 : (size_t)env * P.map_words);
     const GlobalTable<A> tab{P.Q + (size_t)env * P.S * A};
     if (MAP == 1) {
-      auto cls = lds_map([&](int cell) -> uint32_t { return lds[cell >> 4]; });
-      run_env_steps<A>(R, P, env, t0, n_steps, cls, cr, tab);
+      run_env_steps<A>(R, P, env, t0, n_steps, MovesLds<A>{lds, 1}, own_map, cr, tab);
     } else {
-      NearMap cls{};
-      cls.g = P.map + (P.map_shared ? 0 : (size_t)env * P.map_words);
-      cls.W = R.W;
-      cls.H = R.H;
-      run_env_steps<A>(R, P, env, t0, n_steps, cls, cr, tab);
+      const MovesGlobal<A> moves{P.moves + (P.map_shared ? 0 : (size_t)env * P.mv_words)};
+      run_env_steps<A>(R, P, env, t0, n_steps, moves, own_map, cr, tab);
     }
   }
 }
@@ -515,7 +511,6 @@ __global__ __launch_bounds__(LDSW ? 320 : 256) void k_fused_tickets(const Rules 
   const int cap = lds_worker ? kTicketEnvs : 64;
   const unsigned take = lds_worker ? 1u : 2u;
   const size_t table = P.S * A;  // floats per table
-  auto cls = lds_map([&](int cell) -> uint32_t { return my_words[(cell >> 4) * 64 + lane]; });
 
   while (true) {
     unsigned base = 0;
@@ -548,7 +543,8 @@ __global__ __launch_bounds__(LDSW ? 320 : 256) void k_fused_tickets(const Rules 
         else if (FAST)
           run_env_fast<A, false>(R, P, env, t0, n_steps, MovesFromMap<A>{my_words + lane, R.W, R.H}, tab);
         else
-          run_env_steps<A>(R, P, env, t0, n_steps, cls, cr, tab);
+          run_env_steps<A>(R, P, env, t0, n_steps, MovesFromMap<A>{my_words + lane, R.W, R.H},
+                           P.map + (size_t)env * P.map_words, cr, tab);
       }
     } else {
       // tables in: n_here consecutive tables are one contiguous run in HBM
@@ -588,7 +584,8 @@ __global__ __launch_bounds__(LDSW ? 320 : 256) void k_fused_tickets(const Rules 
         }
       } else if (live) {
         const LdsTable<A> tab{tabs + lane * tab_stride};
-        run_env_steps<A>(R, P, env, t0, n_steps, cls, cr, tab);
+        run_env_steps<A>(R, P, env, t0, n_steps, MovesFromMap<A>{my_words + lane, R.W, R.H},
+                         P.map + (size_t)env * P.map_words, cr, tab);
       }
       __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
       __builtin_amdgcn_wave_barrier();
