@@ -4,7 +4,7 @@
 //   s, ep_step, episode : int32    reward : fp32    done, action : uint8
 //   start               : int32 cell index
 //   map                 : 2 bits per cell, 16 cells per uint32, map_words per map
-//   moves               : 2 bits per (cell, action), derived from map (per-env maps only)
+//   moves               : 2 bits per (cell, action), derived from map, mv_words per map
 //   cell_reward         : fp32 per cell (optional)
 //   Q                   : fp32 [table][s][a], one table per env or one shared
 //
@@ -25,7 +25,7 @@ struct Ptrs {
   uint8_t* done;
   uint8_t* action;
   const uint32_t* map;
-  const uint32_t* moves;  // packed move codes of every cell, mv_words per map (or null)
+  const uint32_t* moves;  // packed move codes of every cell, mv_words per map
   const float* cell_reward;
   float* Q;
   const float* eps_tab;
