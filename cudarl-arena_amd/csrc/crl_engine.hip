@@ -216,7 +216,12 @@ struct FusedPlan {
 constexpr size_t kLdsPerWorkgroup = 160 * 1024;  // gfx950
 constexpr int kHybridMinEnvs = 2048;
 
-FusedPlan plan_fused(const crl_engine* e) {
+// Launches shorter than this do not repay moving whole tables into LDS and back
+// (1M envs of config 4, steps per launch -> env-steps/s, plain / hybrid:
+// 32: 2.4e10 / 2.1e10, 48: 2.8e10 / 2.75e10, 64: 3.0e10 / 3.3e10, 100: 3.6e10 / 4.2e10).
+constexpr int kHybridMinSteps = 64;
+
+FusedPlan plan_fused(const crl_engine* e, int n_steps) {
   FusedPlan p{};
   // small batches spread over more compute units with one-wave blocks
   p.block = e->N >= 256 * 512 ? 256 : 64;
@@ -267,7 +272,8 @@ FusedPlan plan_fused(const crl_engine* e) {
     const size_t tables_lds = (size_t)crl::kTicketEnvs * p.tab_stride * 4;
     const long tickets = (e->N + crl::kTicketEnvs - 1) / crl::kTicketEnvs;
     const bool fits = e->K % 4 == 0 && map_lds + lds_wave + tables_lds <= kLdsPerWorkgroup;
-    p.hybrid = fits && (e->fused_variant == 2 || (e->fused_variant == 0 && e->N >= kHybridMinEnvs));
+    p.hybrid = fits && (e->fused_variant == 2 ||
+                        (e->fused_variant == 0 && e->N >= kHybridMinEnvs && n_steps >= kHybridMinSteps));
     if (p.hybrid) {
       p.grid = (int)std::min<long>(kComputeUnits, (tickets + 8) / 9);
       long hbm_waves = std::min<long>(4, std::max<long>(1, resident / (64L * p.grid)));
@@ -877,7 +883,7 @@ int crl_run_fused(crl_engine* e, int32_t n_steps) {
   if (n_steps < 0) return fail(CRL_E_ARG, "negative step count");
   if (n_steps == 0) return CRL_OK;
   if (e->cfg.table_mode == CRL_TABLE_PER_ENV) {
-    const FusedPlan p = plan_fused(e);
+    const FusedPlan p = plan_fused(e, n_steps);
     if (p.tickets) {
       if (e->ticket.ensure(3) != hipSuccess) return fail(CRL_E_ALLOC, "ticket counter allocation failed");
       if (!e->hybrid_opt_in) {
@@ -1078,7 +1084,7 @@ int crl_fused_kernel_info(crl_engine* e, char* name, size_t name_len, int32_t* g
                           int32_t* lds_bytes) {
   if (!e) return fail(CRL_E_ARG, "null engine");
   if (e->cfg.table_mode == CRL_TABLE_PER_ENV) {
-    const FusedPlan p = plan_fused(e);
+    const FusedPlan p = plan_fused(e, 1 << 20);  // the plan of a long launch
     if (name && name_len) snprintf(name, name_len, "%s", p.name);
     if (grid) *grid = p.grid;
     if (block) *block = p.block;

@@ -100,7 +100,8 @@ __device__ __forceinline__ Draw pick_draw(const Philox4 blk, uint64_t t, int A) 
 // ---------------------------------------------------------------------------
 
 // where an env's table lives while it is being stepped
-constexpr int kTouchFloats = 2048;  // tables up to 8 KB are pulled into the caches whole
+constexpr int kTouchFloats = 2048;  // tables up to 8 KB are pulled into the caches whole ...
+constexpr int kTouchMinSteps = 64;  // ... by launches long enough to use most of their lines
 template <int A>
 struct GlobalTable {  // in HBM / the caches
   float* __restrict__ q;
@@ -537,7 +538,7 @@ __global__ __launch_bounds__(LDSW ? 320 : 256) void k_fused_tickets(const Rules 
       __builtin_amdgcn_wave_barrier();
       if (live) {
         const GlobalTable<A> tab{P.Q + (size_t)env * table};
-        tab.touch((int)table);
+        if (n_steps >= kTouchMinSteps) tab.touch((int)table);
         if (kTableMoves)
           run_env_fast<A, false>(R, P, env, t0, n_steps, MovesLds<A>{my_words + lane, 64}, tab);
         else if (FAST)

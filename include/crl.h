@@ -128,7 +128,8 @@ int crl_set_resident_envs(crl_engine* e, int32_t n_envs);
 /* Tuning (no reference counterpart): kernel of crl_run_fused for per-env tables.
  * 0 = automatic, 1 = plain (every wave steps envs against tables in HBM),
  * 2 = hybrid (the last wave of each workgroup steps envs whose whole tables it holds
- * in LDS; used only when 32 tables fit).  Results do not depend on it. */
+ * in LDS; used only when 32 tables fit; automatic picks it for launches of at
+ * least 64 steps).  Results do not depend on it. */
 int crl_set_fused_variant(crl_engine* e, int32_t variant);
 /* How the last hybrid crl_run_fused split the envs between its two kinds of
  * workers (tables in HBM / tables in LDS); both 0 if the plain kernel ran. */
@@ -236,7 +237,8 @@ enum {
 };
 int crl_device_ptr(crl_engine* e, int32_t which, void** out);
 
-/* name and launch geometry of the kernel crl_run_fused uses for this engine */
+/* name and launch geometry of the kernel crl_run_fused uses for this engine on a
+ * long launch (launches of fewer than 64 steps keep every table in HBM) */
 int crl_fused_kernel_info(crl_engine* e, char* name, size_t name_len, int32_t* grid,
                           int32_t* block, int32_t* lds_bytes);
 
