@@ -199,6 +199,7 @@ constexpr int kLdsMapLimitBytes = 64 * 1024;
 constexpr size_t kTableBytesInFlight = (size_t)192 << 20;
 constexpr int kComputeUnits = 256;
 constexpr long kMinEnvsInFlight = kComputeUnits * 3L * 64;  // three waves per compute unit
+constexpr int kInFlightMinSteps = 16;  // shorter launches: 4 steps 6.1e9 -> 6.9e9 with all envs in flight
 
 // launch geometry of the fused per-env kernel
 struct FusedPlan {
@@ -210,6 +211,7 @@ struct FusedPlan {
   bool hybrid;     // ... whose last wave per workgroup steps envs whose tables it holds in LDS
   bool fast;       // the folded loop for the common configuration
   bool moves;      // ... whose table waves read pre-built move codes from LDS
+  bool fixed;      // every pair of tickets has its own wave: dealt by position, no counter
   int tab_stride;  // floats between two tables in LDS
 };
 
@@ -220,6 +222,7 @@ constexpr int kHybridMinEnvs = 2048;
 // (1M envs of config 4, steps per launch -> env-steps/s, plain / hybrid:
 // 32: 2.4e10 / 2.1e10, 48: 2.8e10 / 2.75e10, 64: 3.0e10 / 3.3e10, 100: 3.6e10 / 4.2e10).
 constexpr int kHybridMinSteps = 64;
+constexpr int kStagedMovesMinSteps = 128;
 
 FusedPlan plan_fused(const crl_engine* e, int n_steps) {
   FusedPlan p{};
@@ -249,7 +252,9 @@ FusedPlan plan_fused(const crl_engine* e, int n_steps) {
   if (resident <= 0) {
     const size_t table_bytes = e->K * sizeof(float);
     resident = e->N;
-    if ((size_t)e->N * table_bytes > kTableBytesInFlight)
+    // (a launch of a few steps re-uses no row often enough for that to matter: it
+    // runs with every env in flight)
+    if ((size_t)e->N * table_bytes > kTableBytesInFlight && n_steps >= kInFlightMinSteps)
       resident = std::max<long>(kMinEnvsInFlight, (long)(kTableBytesInFlight / table_bytes));
   }
   p.tickets = p.map_kind == 0;
@@ -295,7 +300,10 @@ FusedPlan plan_fused(const crl_engine* e, int n_steps) {
         p.grid = (int)std::min<long>(std::max<long>(1, resident / 256), (tickets + 7) / 8);
       }
       p.block = 64 * (int)waves;
-      p.moves = p.fast && waves * mv_lds <= kLdsPerWorkgroup;
+      // staging the codes (four times the class map) pays off over a long launch only:
+      // 1M envs of config 4, one step per launch 7.7e9 -> 1.4e10 with class maps, 48 steps 3.6e10 -> 3.7e10
+      p.moves = p.fast && waves * mv_lds <= kLdsPerWorkgroup && n_steps >= kStagedMovesMinSteps;
+      p.fixed = (long)p.grid * waves * 2 >= tickets && n_steps < kHybridMinSteps;  // a wave for every pair of tickets
       p.lds = waves * (p.moves ? mv_lds : map_lds);
     }
   }
@@ -324,7 +332,7 @@ void launch_fused_a(const crl_engine* e, const FusedPlan& p, uint64_t t0, int n)
     unsigned* tk = e->ticket.p;
 #define CRL_LAUNCH_TICKETS(FAST, LDSW, MOVES)                                                       \
   hipLaunchKernelGGL((crl::k_fused_tickets<A, FAST, LDSW, MOVES>), g, b, p.lds, e->stream, R, P, t0, n, \
-                     tk, p.tab_stride)
+                     tk, p.tab_stride, p.fixed ? 1 : 0)
     if (p.fast && p.hybrid)
       CRL_LAUNCH_TICKETS(true, true, false);
     else if (p.fast && p.moves)

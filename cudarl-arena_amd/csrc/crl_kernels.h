@@ -481,14 +481,25 @@ __global__ __launch_bounds__(256) void k_fused_per_env(const Rules R, const Ptrs
 // and derive the codes while their row loads are in flight.
 constexpr int kTicketEnvs = 32;
 
-// `count` envs' words (`wpe` per env, contiguous in HBM) into [word][lane]
+// `count` envs' words (`wpe` per env, contiguous in HBM) into [word][lane]; eight
+// loads in flight per lane (one at a time, a short launch is spent waiting here)
 __device__ __forceinline__ void stage_words(const uint32_t* __restrict__ src, const int count,
                                             const int wpe, const int stride, uint32_t* dst,
                                             const int lane) {
-  for (int i = lane; i < count * wpe; i += 64) {
+  const int total = count * wpe;
+  auto put = [&](int i, uint32_t v) {
     const int e = i / wpe, w = i - e * wpe;
-    dst[w * stride + e] = __builtin_nontemporal_load(src + i);  // read once per launch
+    dst[w * stride + e] = v;
+  };
+  int i0 = 0;
+  for (; i0 + 64 * 8 <= total; i0 += 64 * 8) {
+    uint32_t v[8];
+#pragma unroll
+    for (int u = 0; u < 8; ++u) v[u] = __builtin_nontemporal_load(src + i0 + u * 64 + lane);  // read once per launch
+#pragma unroll
+    for (int u = 0; u < 8; ++u) put(i0 + u * 64 + lane, v[u]);
   }
+  for (int i = i0 + lane; i < total; i += 64) put(i, __builtin_nontemporal_load(src + i));
 }
 
 template <int A, bool FAST, bool LDSW, bool MOVES>
@@ -496,7 +507,8 @@ __global__ __launch_bounds__(LDSW ? 320 : 256) void k_fused_tickets(const Rules 
                                                                      const uint64_t t0,
                                                                      const int n_steps,
                                                                      unsigned* __restrict__ ticket,
-                                                                     const int tab_stride) {
+                                                                     const int tab_stride,
+                                                                     const int fixed_tickets) {
   extern __shared__ uint32_t lds[];
   const int n_waves = (int)(blockDim.x >> 6);  // with LDSW the last one works on LDS tables
   const int lane = threadIdx.x & 63;
@@ -513,16 +525,27 @@ __global__ __launch_bounds__(LDSW ? 320 : 256) void k_fused_tickets(const Rules 
   const unsigned take = lds_worker ? 1u : 2u;
   const size_t table = P.S * A;  // floats per table
 
-  while (true) {
+  // With a wave for every pair of tickets (fixed_tickets: a short launch with all
+  // envs in flight) the tickets are dealt by position: tens of thousands of
+  // atomic draws from one counter would take longer than the few steps.
+  if (fixed_tickets && blockIdx.x == 0 && threadIdx.x == 0) {
+    ticket[1] = (unsigned)P.N;
+    ticket[2] = 0u;
+  }
+  for (bool first = true;; first = false) {
     unsigned base = 0;
-    if (lane == 0) base = atomicAdd(ticket, take);
-    base = __shfl(base, 0);
+    if (fixed_tickets) {
+      base = first ? (blockIdx.x * (unsigned)n_waves + (unsigned)wave) * take : n_tickets;
+    } else {
+      if (lane == 0) base = atomicAdd(ticket, take);
+      base = __shfl(base, 0);
+    }
     if (base >= n_tickets) break;  // every worker gets here: the counter only grows
     const int env0 = (int)base * kTicketEnvs;
     const int n_here = min(cap, P.N - env0);
     const int env = env0 + lane;
     const bool live = lane < n_here;
-    if (lane == 0) atomicAdd(ticket + (lds_worker ? 2 : 1), (unsigned)n_here);  // who did how much
+    if (!fixed_tickets && lane == 0) atomicAdd(ticket + (lds_worker ? 2 : 1), (unsigned)n_here);  // who did how much
 
     // this worker's maps: contiguous in HBM, transposed into [word][lane]
     __builtin_amdgcn_wave_barrier();
