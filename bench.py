@@ -38,7 +38,7 @@ WORKLOADS = {
                name="c3: 65536 envs, shared 64x64 map, one shared table 4096x4, ordered reduction"),
     # traffic: HBM bytes per env-step from rocprofv3 FETCH_SIZE x2.000 + WRITE_SIZE x1.000
     # (profiles/k_fused_tickets_c4.md), valid for the default launch only
-    "c4": dict(n=1 << 20, w=16, h=16, a=4, t=128, steps=1000, warmup=128, bytes=42.25, traffic=31.2,
+    "c4": dict(n=1 << 20, w=16, h=16, a=4, t=128, steps=1000, warmup=128, bytes=42.25, traffic=30.8,
                name="c4: 1048576 envs 16x16, per-env tables 256x4 (4 GB), traps, eps 0.1, T=128"),
     "c5": dict(n=8192, w=256, h=256, a=8, t=1024, steps=1024, warmup=64, bytes=70.0,
                name="c5: 8192 envs 256x256, 8 actions, per-env tables 65536x8 (16 GB), cell rewards"),
