@@ -216,7 +216,6 @@ struct FusedPlan {
 };
 
 constexpr size_t kLdsPerWorkgroup = 160 * 1024;  // gfx950
-constexpr int kHybridMinEnvs = 2048;
 
 // Launches shorter than this do not repay moving whole tables into LDS and back
 // (1M envs of config 4, steps per launch -> env-steps/s, plain / hybrid:
@@ -277,8 +276,12 @@ FusedPlan plan_fused(const crl_engine* e, int n_steps) {
     const size_t tables_lds = (size_t)crl::kTicketEnvs * p.tab_stride * 4;
     const long tickets = (e->N + crl::kTicketEnvs - 1) / crl::kTicketEnvs;
     const bool fits = e->K % 4 == 0 && map_lds + lds_wave + tables_lds <= kLdsPerWorkgroup;
+    // ... and (automatic) when the tables outgrow the caches: while they all fit,
+    // plain waves on every SIMD are faster (16x16 maps, env-steps/s plain / hybrid:
+    // 32,768 envs 5.7e10 / 4.6e10, 65,536 envs 5.5e10 / 6.3e10, 262,144 envs 6.1e10 / 8.1e10)
+    const bool outgrown = (size_t)e->N * e->K * sizeof(float) > kTableBytesInFlight;
     p.hybrid = fits && (e->fused_variant == 2 ||
-                        (e->fused_variant == 0 && e->N >= kHybridMinEnvs && n_steps >= kHybridMinSteps));
+                        (e->fused_variant == 0 && outgrown && n_steps >= kHybridMinSteps));
     if (p.hybrid) {
       p.grid = (int)std::min<long>(kComputeUnits, (tickets + 8) / 9);
       long hbm_waves = std::min<long>(4, std::max<long>(1, resident / (64L * p.grid)));
