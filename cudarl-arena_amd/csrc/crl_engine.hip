@@ -284,7 +284,9 @@ FusedPlan plan_fused(const crl_engine* e, int n_steps) {
                         (e->fused_variant == 0 && outgrown && n_steps >= kHybridMinSteps));
     if (p.hybrid) {
       p.grid = (int)std::min<long>(kComputeUnits, (tickets + 8) / 9);
-      long hbm_waves = std::min<long>(4, std::max<long>(1, resident / (64L * p.grid)));
+      // at most three, so that the LDS wave has a SIMD to itself (1M envs, 8x8 / 12x12
+      // maps: 1.11e11 / 1.00e11 env-steps/s with three table waves, 1.00e11 / 8.4e10 with four)
+      long hbm_waves = std::min<long>(3, std::max<long>(1, resident / (64L * p.grid)));
       while (hbm_waves * map_lds + lds_wave + tables_lds > kLdsPerWorkgroup) --hbm_waves;
       p.block = 64 * ((int)hbm_waves + 1);
       p.lds = hbm_waves * map_lds + lds_wave + tables_lds;
