@@ -181,6 +181,14 @@ __device__ __forceinline__ void row_opaque(Row<8>& r) {
   asm volatile("" : "+v"(r.q0), "+v"(r.q1), "+v"(r.q2), "+v"(r.q3), "+v"(r.q4), "+v"(r.q5), "+v"(r.q6), "+v"(r.q7));
 }
 
+__device__ __forceinline__ Row<4> row_pick(bool c, const Row<4> a, const Row<4> b) {
+  return Row<4>{c ? a.q0 : b.q0, c ? a.q1 : b.q1, c ? a.q2 : b.q2, c ? a.q3 : b.q3};
+}
+__device__ __forceinline__ Row<8> row_pick(bool c, const Row<8> a, const Row<8> b) {
+  return Row<8>{c ? a.q0 : b.q0, c ? a.q1 : b.q1, c ? a.q2 : b.q2, c ? a.q3 : b.q3,
+                c ? a.q4 : b.q4, c ? a.q5 : b.q5, c ? a.q6 : b.q6, c ? a.q7 : b.q7};
+}
+
 // lowest index wins ties (src/q_learning.cu:200-206: strict >)
 __device__ __forceinline__ void amax_step(float v, int i, float& bv, int& bi) {
   const bool gt = v > bv;

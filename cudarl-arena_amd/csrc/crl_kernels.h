@@ -199,6 +199,10 @@ __device__ __forceinline__ void run_env_steps(const Rules& R, const Ptrs& P, con
     start_goal = cell_class_of(own_map[start >> 4], start) == kGoal;
   }
   Philox4 blk = explore_block(R.seed, (uint32_t)env, t0 >> 1);
+  // Epsilon of a per-episode schedule stays in a register and is looked up again
+  // only when an episode of the wave ends: as a load at the top of every step it
+  // was a second round trip to memory per step, in front of the action.
+  float eps = eps_of(R, P.eps_tab, t0, episode);
   const bool track = P.ret_acc != nullptr;
   float ret = track ? P.ret_acc[env] : 0.0f;
   // nothing loaded above is still in flight when the loop starts (a value still in
@@ -206,7 +210,7 @@ __device__ __forceinline__ void run_env_steps(const Rules& R, const Ptrs& P, con
   // operations on every iteration, the previous step's stores included)
   row_opaque(row);
   asm volatile("" : "+v"(ep_step), "+v"(episode), "+v"(reward), "+v"(action), "+v"(ret), "+v"(mv),
-               "+v"(start), "+v"(s), "+v"(on_goal), "+v"(start_goal));
+               "+v"(start), "+v"(s), "+v"(on_goal), "+v"(start_goal), "+v"(eps));
 
   for (int k = 0; k < n_steps; ++k) {
     if (R.max_episodes > 0 && episode >= R.max_episodes) {
@@ -221,7 +225,8 @@ __device__ __forceinline__ void run_env_steps(const Rules& R, const Ptrs& P, con
       d.u = P.u_sup[o];
       d.a = P.a_sup[o];
     }
-    const float eps = eps_of(R, P.eps_tab, t, episode);
+    // indexed by the step: one address for the whole wave, read every step
+    if (R.eps_mode == 1) eps = eps_of(R, P.eps_tab, t, episode);
     const int a = (d.u < eps) ? d.a : row_argmax(row);
 
     // the move (src/kernels.cu:13-66; goal on the resulting cell: src/environment.cu:43)
@@ -258,8 +263,12 @@ __device__ __forceinline__ void run_env_steps(const Rules& R, const Ptrs& P, con
     x = ends ? sx : x + dx;
     y = ends ? sy : y + dy;
     on_goal = ends ? start_goal : on_goal2;
+    // (the second row only when an episode of the wave ends: a request that
+    // nobody needs still takes its turn in the memory pipeline)
+    const bool any_ends = __builtin_amdgcn_ballot_w64(ends) != 0;
     const Row<A> row2 = tab.load(s2);
-    const Row<A> row_next = tab.load(s);
+    Row<A> row_restart{};
+    if (any_ends) row_restart = tab.load(s);
     mv = moves.at(s, x, y);
     // the next step's draws depend on nothing: the Philox rounds run while the
     // loads are in flight
@@ -268,7 +277,7 @@ __device__ __forceinline__ void run_env_steps(const Rules& R, const Ptrs& P, con
     const float qn = td_value(row_get(row, a), reward, m, R.lr, R.gamma);
     tab.store(s0, a, qn);
     // the value just written, patched in from registers
-    row = row_set(row_next, s == s0 ? a : -1, qn);
+    row = row_set(row_pick(ends, row_restart, row2), s == s0 ? a : -1, qn);
 
     action = a;
     ret = ret + reward;
@@ -283,6 +292,10 @@ __device__ __forceinline__ void run_env_steps(const Rules& R, const Ptrs& P, con
     ret = ends ? 0.0f : ret;
     ep_step = ends ? 0 : ep_step;
     episode += ends ? 1 : 0;
+    if (R.eps_mode >= 2 && any_ends) {
+      eps = eps_of(R, P.eps_tab, t, episode);
+      asm volatile("" : "+v"(eps));  // arrived before the loop goes round
+    }
   }
 
   P.s[env] = s;
