@@ -267,14 +267,17 @@ FusedPlan plan_fused(const crl_engine* e, int n_steps) {
     }
   }
   p.tickets = p.map_kind == 0;
+  const crl_config& c = e->cfg;
+  // what the folded loop leaves out altogether ...
+  const bool foldable = c.goal_mode == CRL_GOAL_ON_TARGET && c.auto_reset == 1 && c.max_mode == CRL_MAX_TRUE &&
+                        e->trace_n == 0 && e->sup_n == 0 && c.max_episodes == 0 && c.track_returns == 0 &&
+                        e->mv_words > 0;
   if (!p.tickets) {
     p.grid = (int)std::min<long>((e->N + p.block - 1) / p.block, std::max<long>(1, resident / p.block));
+    // ... its variant for large or shared maps takes per-cell rewards and per-episode epsilon
+    p.fast = foldable && c.eps_mode != CRL_EPS_STEP_MULT && c.table_mode != CRL_TABLE_SHARED;
   } else {
-    const crl_config& c = e->cfg;
-    p.fast = c.eps_mode == CRL_EPS_FIXED && c.reward_flags == 0 && c.goal_mode == CRL_GOAL_ON_TARGET &&
-             c.auto_reset == 1 && c.max_mode == CRL_MAX_TRUE && e->trace_n == 0 && e->sup_n == 0 &&
-             c.max_episodes == 0 && c.track_returns == 0;
-    p.fast = p.fast && e->mv_words > 0;
+    p.fast = foldable && c.eps_mode == CRL_EPS_FIXED && c.reward_flags == 0;
     // Hybrid workgroups when 32 whole tables (padded by one row against bank
     // conflicts), the LDS wave's maps and at least one table wave's maps fit into
     // LDS.  One workgroup per compute unit (the LDS holds no second one); the envs
@@ -322,10 +325,12 @@ FusedPlan plan_fused(const crl_engine* e, int n_steps) {
       p.lds = waves * (p.moves ? mv_lds : map_lds);
     }
   }
-  static const char* names[2][3] = {
-      {"k_fused_per_env<4,0>", "k_fused_per_env<4,1>", "k_fused_per_env<4,2>"},
-      {"k_fused_per_env<8,0>", "k_fused_per_env<8,1>", "k_fused_per_env<8,2>"}};
-  p.name = names[e->A == 8][p.map_kind];
+  static const char* names[2][2][3] = {
+      {{"k_fused_per_env<4,0>", "k_fused_per_env<4,1,general>", "k_fused_per_env<4,2,general>"},
+       {"k_fused_per_env<4,0>", "k_fused_per_env<4,1,fast>", "k_fused_per_env<4,2,fast>"}},
+      {{"k_fused_per_env<8,0>", "k_fused_per_env<8,1,general>", "k_fused_per_env<8,2,general>"},
+       {"k_fused_per_env<8,0>", "k_fused_per_env<8,1,fast>", "k_fused_per_env<8,2,fast>"}}};
+  p.name = names[e->A == 8][p.fast][p.map_kind];
   if (p.tickets) {
     static const char* tnames[2][2][2] = {
         {{"k_fused_tickets<4,general,hbm>", "k_fused_tickets<4,general,hbm+lds>"},
@@ -361,16 +366,18 @@ void launch_fused_a(const crl_engine* e, const FusedPlan& p, uint64_t t0, int n)
 #undef CRL_LAUNCH_TICKETS
     return;
   }
-  switch (p.map_kind) {
-    case 1:
-      hipLaunchKernelGGL((crl::k_fused_per_env<A, 1>), dim3(p.grid), dim3(p.block), p.lds, e->stream,
-                         R, P, t0, n);
-      break;
-    default:
-      hipLaunchKernelGGL((crl::k_fused_per_env<A, 2>), dim3(p.grid), dim3(p.block), 0, e->stream, R, P,
-                         t0, n);
-      break;
-  }
+#define CRL_LAUNCH_PER_ENV(MAP, FAST)                                                                 \
+  hipLaunchKernelGGL((crl::k_fused_per_env<A, MAP, FAST>), dim3(p.grid), dim3(p.block),               \
+                     MAP == 1 ? p.lds : 0, e->stream, R, P, t0, n)
+  if (p.map_kind == 1 && p.fast)
+    CRL_LAUNCH_PER_ENV(1, true);
+  else if (p.map_kind == 1)
+    CRL_LAUNCH_PER_ENV(1, false);
+  else if (p.fast)
+    CRL_LAUNCH_PER_ENV(2, true);
+  else
+    CRL_LAUNCH_PER_ENV(2, false);
+#undef CRL_LAUNCH_PER_ENV
 }
 
 constexpr size_t kHandoffLimitBytes = (size_t)128 << 20;

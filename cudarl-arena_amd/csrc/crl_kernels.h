@@ -323,16 +323,29 @@ __device__ __forceinline__ void run_env_steps(const Rules& R, const Ptrs& P, con
 // rounds, the most expensive stretch of a step that waits for no memory: one
 // lane computes the block of the next two steps, the other the block after, and
 // they swap, so the rounds run every fourth step instead of every second.
-template <int A, bool PAIR, class Table, class Moves>
+//
+// RICH adds the two things that configurations with large maps bring along and
+// that cost one more request per step at most: per-cell rewards (`cr`, may be
+// null) and an epsilon that follows the env's episode count.  The threshold
+// stays in a register and is looked up again only when an episode of the wave
+// ends, and so is the row of the start cell: with long episodes both are rare.
+template <int A, bool PAIR, bool RICH, class Table, class Moves>
 __device__ __forceinline__ void run_env_fast(const Rules& R, const Ptrs& P, const int env,
                                              const uint64_t t0, const int n_steps, const Moves moves,
-                                             const Table tab) {
+                                             const float* __restrict__ cr, const Table tab) {
   const int W = R.W, T = R.episode_len;
   const float lr = R.lr, gamma = R.gamma;
   // u01(w) < eps  <=>  (w >> 8) < eps * 2^24, both sides exact: an integer compare
-  const float scaled = ceilf(R.eps0 * 16777216.0f);
-  const uint32_t explore_below = !(scaled > 0.0f) ? 0u : scaled >= 16777216.0f ? (1u << 24) : (uint32_t)scaled;
-  const float r_step = R.step_reward, r_goal = R.goal_reward, r_trap = R.trap_reward;
+  auto threshold = [](float eps) -> uint32_t {
+    const float scaled = ceilf(eps * 16777216.0f);
+    return !(scaled > 0.0f) ? 0u : scaled >= 16777216.0f ? (1u << 24) : (uint32_t)scaled;
+  };
+  uint32_t explore_below = threshold(R.eps0);
+  float r_step = R.step_reward, r_goal = R.goal_reward, r_trap = R.trap_reward;
+  if (RICH) asm volatile("" : "+v"(r_step), "+v"(r_goal), "+v"(r_trap));  // plain values: no select of loads
+  const bool cells = RICH && cr != nullptr;
+  const bool base_cells = cells && (R.reward_flags & 2) != 0;
+  const bool scheduled = RICH && R.eps_mode >= 2;
   int start = P.start[env];
   const int sx = start % W, sy = start / W;
   int s = P.s[env];
@@ -344,6 +357,7 @@ __device__ __forceinline__ void run_env_fast(const Rules& R, const Ptrs& P, cons
   bool hit = false;
   Row<A> row = tab.load(s);
   uint32_t mv = moves.at(s, x, y);
+  if (scheduled) explore_below = threshold(eps_of(R, P.eps_tab, t0, episode));
   const int lane = (int)__lane_id();
   const bool upper = PAIR && lane >= 32;
   // own block, and (PAIR) the partner lane's: {blk, nxt} = the next two blocks
@@ -377,6 +391,7 @@ __device__ __forceinline__ void run_env_fast(const Rules& R, const Ptrs& P, cons
   // included
   row_opaque(row);
   asm volatile("" : "+v"(ep_step), "+v"(episode), "+v"(mv), "+v"(start), "+v"(s));
+  if (RICH) asm volatile("" : "+v"(explore_below));
 
   for (int k = 0; k < n_steps; ++k) {
     const uint32_t w0 = odd ? blk.w2 : blk.w0;
@@ -389,11 +404,19 @@ __device__ __forceinline__ void run_env_fast(const Rules& R, const Ptrs& P, cons
     const bool moved = code < (uint32_t)kTrap;
     int dx, dy;
     action_delta(a, A, dx, dy);
+    hit = code == (uint32_t)kGoal;
+    const bool trap = code == (uint32_t)kTrap;
+    reward = hit ? r_goal : (trap ? r_trap : r_step);
+    float by_cell = 0.0f;
+    if (RICH && cells) {
+      // the goal pays on the goal cell (where the move ends), the trap on the
+      // cell it guards, anything else where the move ends: one load at one index
+      const int tgt = s + __mul24(dy, W) + dx;
+      by_cell = cr[trap ? tgt : (moved ? tgt : s)];
+    }
     dx = moved ? dx : 0;
     dy = moved ? dy : 0;
     const int s2 = s + __mul24(dy, W) + dx;
-    hit = code == (uint32_t)kGoal;
-    reward = hit ? r_goal : (code == (uint32_t)kTrap ? r_trap : r_step);
 
     // Two rows are asked for together: the one of the cell the move ends on (for
     // the TD target) and the one of the cell the env acts from next - the same
@@ -405,7 +428,9 @@ __device__ __forceinline__ void run_env_fast(const Rules& R, const Ptrs& P, cons
     const bool ends = hit || (T > 0 && ep_step >= T);
     const int s_next = ends ? start : s2;
     const Row<A> row2 = tab.load(s2);
-    const Row<A> row_next = tab.load(s_next);
+    Row<A> row_next{};
+    const bool any_ends = !RICH || __builtin_amdgcn_ballot_w64(ends) != 0;
+    if (any_ends) row_next = tab.load(s_next);
     x = ends ? sx : x + dx;
     y = ends ? sy : y + dy;
     mv = moves.at(s_next, x, y);
@@ -421,17 +446,22 @@ __device__ __forceinline__ void run_env_fast(const Rules& R, const Ptrs& P, cons
         have_nxt = true;
       }
     }
+    if (RICH) reward = (cells && (hit || trap || base_cells)) ? by_cell : reward;
     const float m = row_max(row2, hit, 0);
     const float qn = td_value(row_get(row, a), reward, m, lr, gamma);
     tab.store(s, a, qn);
 
     // the cell to act from next, with the value just written patched in from registers
-    row = row_set(row_next, s_next == s ? a : -1, qn);
+    row = row_set(RICH ? row_pick(ends, row_next, row2) : row_next, s_next == s ? a : -1, qn);
     ep_step = ends ? 0 : ep_step;
     episode += ends ? 1 : 0;
     s = s_next;
     action = a;
     odd = !odd;
+    if (RICH && scheduled && any_ends) {
+      explore_below = threshold(eps_of(R, P.eps_tab, t0, episode));
+      asm volatile("" : "+v"(explore_below));  // arrived before the loop goes round
+    }
   }
 
   P.s[env] = s;
@@ -446,7 +476,7 @@ __device__ __forceinline__ void run_env_fast(const Rules& R, const Ptrs& P, cons
 // in LDS) or too large for LDS (MAP = 2: move codes read from global memory, one
 // load per step).  A block takes chunks blockIdx, blockIdx + gridDim, ... and runs
 // each for all n_steps.
-template <int A, int MAP>
+template <int A, int MAP, bool FAST>
 __global__ __launch_bounds__(256) void k_fused_per_env(const Rules R, const Ptrs P,
                                                         const uint64_t t0, const int n_steps) {
   extern __shared__ uint32_t lds[];
@@ -466,10 +496,16 @@ __global__ __launch_bounds__(256) void k_fused_per_env(const Rules R, const Ptrs
     const uint32_t* own_map = P.map + (P.map_shared ? 0 : (size_t)env * P.map_words);
     const GlobalTable<A> tab{P.Q + (size_t)env * P.S * A};
     if (MAP == 1) {
-      run_env_steps<A>(R, P, env, t0, n_steps, MovesLds<A>{lds, 1}, own_map, cr, tab);
+      if (FAST)
+        run_env_fast<A, false, true>(R, P, env, t0, n_steps, MovesLds<A>{lds, 1}, cr, tab);
+      else
+        run_env_steps<A>(R, P, env, t0, n_steps, MovesLds<A>{lds, 1}, own_map, cr, tab);
     } else {
       const MovesGlobal<A> moves{P.moves + (P.map_shared ? 0 : (size_t)env * P.mv_words)};
-      run_env_steps<A>(R, P, env, t0, n_steps, moves, own_map, cr, tab);
+      if (FAST)
+        run_env_fast<A, false, true>(R, P, env, t0, n_steps, moves, cr, tab);
+      else
+        run_env_steps<A>(R, P, env, t0, n_steps, moves, own_map, cr, tab);
     }
   }
 }
@@ -576,9 +612,9 @@ __global__ __launch_bounds__(LDSW ? 320 : 256) void k_fused_tickets(const Rules 
         const GlobalTable<A> tab{P.Q + (size_t)env * table};
         if (n_steps >= kTouchMinSteps) tab.touch((int)table);
         if (kTableMoves)
-          run_env_fast<A, false>(R, P, env, t0, n_steps, MovesLds<A>{my_words + lane, 64}, tab);
+          run_env_fast<A, false, false>(R, P, env, t0, n_steps, MovesLds<A>{my_words + lane, 64}, nullptr, tab);
         else if (FAST)
-          run_env_fast<A, false>(R, P, env, t0, n_steps, MovesFromMap<A>{my_words + lane, R.W, R.H}, tab);
+          run_env_fast<A, false, false>(R, P, env, t0, n_steps, MovesFromMap<A>{my_words + lane, R.W, R.H}, nullptr, tab);
         else
           run_env_steps<A>(R, P, env, t0, n_steps, MovesFromMap<A>{my_words + lane, R.W, R.H},
                            P.map + (size_t)env * P.map_words, cr, tab);
@@ -617,7 +653,7 @@ __global__ __launch_bounds__(LDSW ? 320 : 256) void k_fused_tickets(const Rules 
         const int l = lane & (kTicketEnvs - 1);
         if (l < n_here) {
           const LdsTable<A> tab{tabs + l * tab_stride};
-          run_env_fast<A, true>(R, P, env0 + l, t0, n_steps, MovesLds<A>{my_words + l, kTicketEnvs}, tab);
+          run_env_fast<A, true, false>(R, P, env0 + l, t0, n_steps, MovesLds<A>{my_words + l, kTicketEnvs}, nullptr, tab);
         }
       } else if (live) {
         const LdsTable<A> tab{tabs + lane * tab_stride};

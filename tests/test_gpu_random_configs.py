@@ -53,6 +53,49 @@ def test_random_configs_folded_loop(gpu, oracle, seed):
         assert same(q, st, Q, ost), (seed, case, name, A, W, H, N, T, steps, t0, eps, variant, resident)
 
 
+@pytest.mark.parametrize("seed", [4, 5])
+def test_random_configs_folded_loop_large_or_shared_maps(gpu, oracle, seed):
+    """The folded loop's variant for maps that are shared or too large for LDS:
+    per-cell rewards (all three reward sources), epsilon fixed or following the
+    env's episode count, 4 and 8 actions, short and long episodes."""
+    rng = np.random.default_rng(seed)
+    for case in range(40):
+        A = int(rng.choice([4, 8]))
+        shared_map = rng.random() < 0.5
+        big = rng.random() < (0.3 if shared_map else 1.0)  # per-env maps reach this kernel only when large
+        W, H = (int(rng.integers(65, 100)) if big else int(rng.integers(2, 40)) for _ in range(2))
+        N = int(rng.choice([1, 63, 64, 65, 300, 1000] if big else [1, 33, 257, 700, 3000]))
+        T = int(rng.choice([0, 1, 2, 9, 40, 400]))
+        steps, t0 = int(rng.integers(1, 160)), int(rng.integers(0, 5))
+        eps_mode, span = int(rng.choice([0, 2, 3])), int(rng.integers(1, 30))
+        flags = int(rng.choice([0, gpu.REWARD_CELLS, gpu.REWARD_CELLS | gpu.REWARD_BASE_CELLS]))
+        map_seed = int(rng.integers(0, 1 << 30))
+        n_maps = 1 if shared_map else N
+        if flags:
+            cls, start, cr = gpu.gen_maps_noise(map_seed, n_maps, W, H, 8, 0.2, 0.3, 5.0)
+            start = np.resize(start, N).astype(np.int32)
+        else:
+            cls, start = gpu.gen_maps_bernoulli(map_seed, n_maps, N, W, H, 0.15, 0.05)
+            cr = None
+        cfg = gpu.make_config(N, W, H, n_actions=A, map_mode=gpu.MAP_SHARED if shared_map else gpu.MAP_PER_ENV,
+                              episode_len=T, lr=0.2, gamma=0.9, reward_flags=flags, eps_mode=eps_mode,
+                              eps0=float(rng.choice([0.0, 0.3, 0.6, 1.0])), eps_decay=0.9, eps_end=0.05,
+                              eps_span=span, seed=map_seed, trap_reward=-0.5)
+        with gpu.Engine(cfg, 0) as eng:
+            eng.set_maps(cls, start, cr)
+            eng.step_count = t0
+            name = eng.fused_kernel_info()["name"]
+            third = steps // 3
+            for c in (third, steps - 2 * third, third):
+                eng.run_fused(c)
+            q, st = eng.q_get(0, N), eng.get_state()
+        Q = np.zeros((N, W * H, A), np.float32)
+        ost = oracle.new_state(cfg, start)
+        oracle.run(cfg, cls, cr, start, Q, ost, t0, steps)
+        assert name.startswith("k_fused_per_env") and "fast" in name, name
+        assert same(q, st, Q, ost), (seed, case, name, A, W, H, N, T, steps, t0, eps_mode, flags, shared_map)
+
+
 @pytest.mark.parametrize("seed", [1, 7])
 def test_random_configs_general(gpu, oracle, seed):
     """Everything else: shared tables and maps, maps too large for LDS, per-cell
