@@ -475,21 +475,28 @@ __device__ __forceinline__ void run_env_fast(const Rules& R, const Ptrs& P, cons
 // Per-env tables whose maps are shared (MAP = 1: the one map's move codes staged
 // in LDS) or too large for LDS (MAP = 2: move codes read from global memory, one
 // load per step).  A block takes chunks blockIdx, blockIdx + gridDim, ... and runs
-// each for all n_steps.
-template <int A, int MAP, bool FAST>
+// each for all n_steps.  MODE 0: the general loop, 1: the folded loop, 2: the
+// folded loop with two lanes per env (a batch too small to give every SIMD a wave
+// of 64 envs: twice the waves, each with half the distinct addresses per request,
+// and the Philox rounds shared between the lanes of a pair).
+template <int A, int MAP, int MODE>
 __global__ __launch_bounds__(256) void k_fused_per_env(const Rules R, const Ptrs P,
                                                         const uint64_t t0, const int n_steps) {
+  constexpr bool FAST = MODE >= 1;
+  constexpr bool PAIR = MODE == 2;  // two lanes per env: lanes l and l + 32 of a wave
   extern __shared__ uint32_t lds[];
   const int tid = threadIdx.x;
   const int bdim = blockDim.x;
-  const int n_chunks = (P.N + bdim - 1) / bdim;
+  const int envs_per_block = PAIR ? bdim >> 1 : bdim;
+  const int n_chunks = (P.N + envs_per_block - 1) / envs_per_block;
+  const int slot = PAIR ? ((tid >> 6) << 5) + (tid & 31) : tid;
 
   if (MAP == 1) {
     for (int i = tid; i < P.mv_words; i += bdim) lds[i] = P.moves[i];
     __syncthreads();
   }
   for (int chunk = blockIdx.x; chunk < n_chunks; chunk += gridDim.x) {
-    const int env = chunk * bdim + tid;
+    const int env = chunk * envs_per_block + slot;
     if (env >= P.N) continue;
     const float* cr =
         P.cell_reward ? P.cell_reward + (P.map_shared ? 0 : (size_t)env * P.S) : nullptr;
@@ -497,13 +504,13 @@ __global__ __launch_bounds__(256) void k_fused_per_env(const Rules R, const Ptrs
     const GlobalTable<A> tab{P.Q + (size_t)env * P.S * A};
     if (MAP == 1) {
       if (FAST)
-        run_env_fast<A, false, true>(R, P, env, t0, n_steps, MovesLds<A>{lds, 1}, cr, tab);
+        run_env_fast<A, PAIR, true>(R, P, env, t0, n_steps, MovesLds<A>{lds, 1}, cr, tab);
       else
         run_env_steps<A>(R, P, env, t0, n_steps, MovesLds<A>{lds, 1}, own_map, cr, tab);
     } else {
       const MovesGlobal<A> moves{P.moves + (P.map_shared ? 0 : (size_t)env * P.mv_words)};
       if (FAST)
-        run_env_fast<A, false, true>(R, P, env, t0, n_steps, moves, cr, tab);
+        run_env_fast<A, PAIR, true>(R, P, env, t0, n_steps, moves, cr, tab);
       else
         run_env_steps<A>(R, P, env, t0, n_steps, moves, own_map, cr, tab);
     }

@@ -64,7 +64,8 @@ def test_random_configs_folded_loop_large_or_shared_maps(gpu, oracle, seed):
         shared_map = rng.random() < 0.5
         big = rng.random() < (0.3 if shared_map else 1.0)  # per-env maps reach this kernel only when large
         W, H = (int(rng.integers(65, 100)) if big else int(rng.integers(2, 40)) for _ in range(2))
-        N = int(rng.choice([1, 63, 64, 65, 300, 1000] if big else [1, 33, 257, 700, 3000]))
+        # (up to 16,384 envs the kernel gives every env two lanes)
+        N = int(rng.choice([1, 63, 64, 65, 300, 1000] if big else [1, 33, 257, 700, 3000, 17000]))
         T = int(rng.choice([0, 1, 2, 9, 40, 400]))
         steps, t0 = int(rng.integers(1, 160)), int(rng.integers(0, 5))
         eps_mode, span = int(rng.choice([0, 2, 3])), int(rng.integers(1, 30))
