@@ -185,7 +185,7 @@ def main():
     ap.add_argument("--probe-copy", type=int, default=0, metavar="MIB",
                     help="only run one plain copy kernel of this many MiB (calibrates rocprofv3 counters)")
     ap.add_argument("--no-cpu", action="store_true", help="skip the cpu_baseline leg")
-    ap.add_argument("--no-also", action="store_true", help="skip the short c2/c3 side measurements")
+    ap.add_argument("--no-also", action="store_true", help="skip the short c2/c3/c5 side measurements")
     args = ap.parse_args()
     if args.gpus != 1:
         raise SystemExit("bench.py: this build runs on ONE GPU (envs shard trivially, but no second "
@@ -246,7 +246,7 @@ def main():
                                          % (min(n_sample, g["n"]), cpu_steps, dt, cores)}
     if not args.no_also and not args.envs:
         also = {}
-        for k2, s2, w2 in (("c3", 300, 20), ("c2", 4000, 256)):
+        for k2, s2, w2 in (("c3", 300, 20), ("c2", 4000, 256), ("c5", 1024, 64)):
             if k2 == key:
                 continue
             r = time_gpu(k2, s2, w2)
