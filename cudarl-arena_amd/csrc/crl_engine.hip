@@ -326,7 +326,14 @@ FusedPlan plan_fused(const crl_engine* e, int n_steps) {
       // staging the codes (four times the class map) pays off over a long launch only:
       // 1M envs of config 4, one step per launch 7.7e9 -> 1.4e10 with class maps, 48 steps 3.6e10 -> 3.7e10
       p.moves = p.fast && waves * mv_lds <= kLdsPerWorkgroup && n_steps >= kStagedMovesMinSteps;
-      p.fixed = (long)p.grid * waves * 2 >= tickets && n_steps < kHybridMinSteps;  // a wave for every pair of tickets
+      // Few enough envs that 32-env waves still find a SIMD each: one ticket per wave,
+      // two lanes per env - half the distinct addresses per request and the Philox
+      // rounds shared by the pair (32x32 maps: 4096 envs +10 %, 8192 +8 %, 16,384 +0 %)
+      if (p.moves && waves == 1 && tickets <= 2 * kComputeUnits) {
+        p.pair = true;
+        p.grid = (int)std::min<long>(std::max<long>(1, resident / 32), tickets);
+      }
+      p.fixed = (long)p.grid * waves * (p.pair ? 1 : 2) >= tickets && n_steps < kHybridMinSteps;  // a wave for every pair of tickets
       p.lds = waves * (p.moves ? mv_lds : map_lds);
     }
   }
@@ -359,7 +366,7 @@ void launch_fused_a(const crl_engine* e, const FusedPlan& p, uint64_t t0, int n)
     unsigned* tk = e->ticket.p;
 #define CRL_LAUNCH_TICKETS(FAST, LDSW, MOVES)                                                       \
   hipLaunchKernelGGL((crl::k_fused_tickets<A, FAST, LDSW, MOVES>), g, b, p.lds, e->stream, R, P, t0, n, \
-                     tk, p.tab_stride, p.fixed ? 1 : 0)
+                     tk, p.tab_stride, p.fixed ? 1 : 0, p.pair ? 1 : 0)
     if (p.fast && p.hybrid)
       CRL_LAUNCH_TICKETS(true, true, false);
     else if (p.fast && p.moves)

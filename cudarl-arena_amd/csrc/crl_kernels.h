@@ -564,7 +564,8 @@ __global__ __launch_bounds__(LDSW ? 320 : 256) void k_fused_tickets(const Rules 
                                                                      const int n_steps,
                                                                      unsigned* __restrict__ ticket,
                                                                      const int tab_stride,
-                                                                     const int fixed_tickets) {
+                                                                     const int fixed_tickets,
+                                                                     const int pair_tables) {
   extern __shared__ uint32_t lds[];
   const int n_waves = (int)(blockDim.x >> 6);  // with LDSW the last one works on LDS tables
   const int lane = threadIdx.x & 63;
@@ -577,8 +578,10 @@ __global__ __launch_bounds__(LDSW ? 320 : 256) void k_fused_tickets(const Rules 
   uint32_t* my_words = lds + wave * slice;  // (the LDS wave is the last one)
   float* tabs = reinterpret_cast<float*>(lds + (n_waves - 1) * slice + lds_slice);
   const unsigned n_tickets = (unsigned)((P.N + kTicketEnvs - 1) / kTicketEnvs);
-  const int cap = lds_worker ? kTicketEnvs : 64;
-  const unsigned take = lds_worker ? 1u : 2u;
+  // (pair_tables: the table waves, too, take one ticket and give every env two lanes)
+  const bool thin = lds_worker || (FAST && MOVES && pair_tables);
+  const int cap = thin ? kTicketEnvs : 64;
+  const unsigned take = thin ? 1u : 2u;
   const size_t table = P.S * A;  // floats per table
 
   // With a wave for every pair of tickets (fixed_tickets: a short launch with all
@@ -615,7 +618,15 @@ __global__ __launch_bounds__(LDSW ? 320 : 256) void k_fused_tickets(const Rules 
     if (!lds_worker) {
       __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
       __builtin_amdgcn_wave_barrier();
-      if (live) {
+      if (kTableMoves && pair_tables) {
+        const int l = lane & (kTicketEnvs - 1);
+        if (l < n_here) {
+          const GlobalTable<A> tab{P.Q + (size_t)(env0 + l) * table};
+          if (n_steps >= kTouchMinSteps) tab.touch((int)table);
+          run_env_fast<A, true, false>(R, P, env0 + l, t0, n_steps, MovesLds<A>{my_words + l, kTicketEnvs},
+                                       nullptr, tab);
+        }
+      } else if (live) {
         const GlobalTable<A> tab{P.Q + (size_t)env * table};
         if (n_steps >= kTouchMinSteps) tab.touch((int)table);
         if (kTableMoves)

@@ -170,12 +170,14 @@ def test_fused_fast_loop_short_launches_no_time_limit(gpu, oracle, variant):
 
 
 @pytest.mark.parametrize("variant,resident", [(1, 0), (1, 192), (2, 0)])
-@pytest.mark.parametrize("N,W,H,A", [(2500, 16, 16, 8), (300, 9, 6, 8), (2100, 7, 5, 4), (130, 33, 31, 4)])
+@pytest.mark.parametrize("N,W,H,A", [(2500, 16, 16, 8), (300, 9, 6, 8), (2100, 7, 5, 4), (130, 33, 31, 4),
+                                     (17000, 9, 6, 4)])
 def test_fused_fast_loop_move_codes(gpu, oracle, variant, resident, N, W, H, A):
     """The folded loop works on per-cell move codes (what each action does from a
     cell) instead of map lookups and bounds tests: pre-built codes staged in LDS
-    (plain kernel, LDS wave of the hybrid one) or derived from the class map
-    (table waves of the hybrid one), with 4 and 8 actions, on grids whose width is
+    (plain kernel - with two lanes per env up to 16,384 envs, one beyond - and the
+    LDS wave of the hybrid one) or derived from the class map (table waves of the
+    hybrid one), with 4 and 8 actions, on grids whose width is
     no multiple of the 16 cells of a map word, with walls, traps and goals on the
     edges."""
     cls, start = gpu.gen_maps_bernoulli(43, N, N, W, H, 0.2, 0.05)
