@@ -213,6 +213,7 @@ struct FusedPlan {
   bool moves;      // ... whose table waves read pre-built move codes from LDS
   bool fixed;      // every pair of tickets has its own wave: dealt by position, no counter
   bool pair;       // per-env kernel: two lanes per env
+  bool rich;       // ticket kernel: the folded loop's variant with per-cell rewards / per-episode epsilon
   int tab_stride;  // floats between two tables in LDS
 };
 
@@ -282,7 +283,8 @@ FusedPlan plan_fused(const crl_engine* e, int n_steps) {
     p.pair = p.fast && (e->N + 63) / 64 <= kComputeUnits;
     if (p.pair) p.grid = (int)std::min<long>((e->N + p.block / 2 - 1) / (p.block / 2), std::max<long>(1, 2 * resident / p.block));
   } else {
-    p.fast = foldable && c.eps_mode == CRL_EPS_FIXED && c.reward_flags == 0;
+    p.rich = foldable && c.eps_mode != CRL_EPS_STEP_MULT && !(c.eps_mode == CRL_EPS_FIXED && c.reward_flags == 0);
+    p.fast = foldable && c.eps_mode != CRL_EPS_STEP_MULT;
     // Hybrid workgroups when 32 whole tables (padded by one row against bank
     // conflicts), the LDS wave's maps and at least one table wave's maps fit into
     // LDS.  One workgroup per compute unit (the LDS holds no second one); the envs
@@ -293,7 +295,9 @@ FusedPlan plan_fused(const crl_engine* e, int n_steps) {
     const size_t lds_wave = p.fast ? (size_t)e->mv_words * crl::kTicketEnvs * 4 : map_lds;
     const size_t tables_lds = (size_t)crl::kTicketEnvs * p.tab_stride * 4;
     const long tickets = (e->N + crl::kTicketEnvs - 1) / crl::kTicketEnvs;
-    const bool fits = e->K % 4 == 0 && map_lds + lds_wave + tables_lds <= kLdsPerWorkgroup;
+    // (not with per-cell rewards: they would stay in HBM, one request per step, and
+    // a worker that waits for memory every step has no use for tables in LDS)
+    const bool fits = e->K % 4 == 0 && map_lds + lds_wave + tables_lds <= kLdsPerWorkgroup && !p.rich;
     // ... and (automatic) when the tables outgrow the caches: while they all fit,
     // plain waves on every SIMD are faster (16x16 maps, env-steps/s plain / hybrid:
     // 32,768 envs 5.7e10 / 4.6e10, 65,536 envs 5.5e10 / 6.3e10, 262,144 envs 6.1e10 / 8.1e10)
@@ -346,12 +350,14 @@ FusedPlan plan_fused(const crl_engine* e, int n_steps) {
        {"k_fused_per_env<8,0>", "k_fused_per_env<8,1,fast,pairs>", "k_fused_per_env<8,2,fast,pairs>"}}};
   p.name = names[e->A == 8][!p.fast ? 0 : p.pair ? 2 : 1][p.map_kind];
   if (p.tickets) {
-    static const char* tnames[2][2][2] = {
+    static const char* tnames[2][3][2] = {
         {{"k_fused_tickets<4,general,hbm>", "k_fused_tickets<4,general,hbm+lds>"},
-         {"k_fused_tickets<4,fast,hbm>", "k_fused_tickets<4,fast,hbm+lds>"}},
+         {"k_fused_tickets<4,fast,hbm>", "k_fused_tickets<4,fast,hbm+lds>"},
+         {"k_fused_tickets<4,fast+,hbm>", "k_fused_tickets<4,fast+,hbm>"}},
         {{"k_fused_tickets<8,general,hbm>", "k_fused_tickets<8,general,hbm+lds>"},
-         {"k_fused_tickets<8,fast,hbm>", "k_fused_tickets<8,fast,hbm+lds>"}}};
-    p.name = tnames[e->A == 8][p.fast][p.hybrid];
+         {"k_fused_tickets<8,fast,hbm>", "k_fused_tickets<8,fast,hbm+lds>"},
+         {"k_fused_tickets<8,fast+,hbm>", "k_fused_tickets<8,fast+,hbm>"}}};
+    p.name = tnames[e->A == 8][p.rich ? 2 : p.fast ? 1 : 0][p.hybrid];
   }
   return p;
 }
@@ -364,19 +370,23 @@ void launch_fused_a(const crl_engine* e, const FusedPlan& p, uint64_t t0, int n)
     hipLaunchKernelGGL(crl::k_fill_u32, dim3(1), dim3(64), 0, e->stream, e->ticket.p, 0u, 3);
     const dim3 g(p.grid), b(p.block);
     unsigned* tk = e->ticket.p;
-#define CRL_LAUNCH_TICKETS(FAST, LDSW, MOVES)                                                       \
-  hipLaunchKernelGGL((crl::k_fused_tickets<A, FAST, LDSW, MOVES>), g, b, p.lds, e->stream, R, P, t0, n, \
+#define CRL_LAUNCH_TICKETS(MODE, LDSW, MOVES)                                                       \
+  hipLaunchKernelGGL((crl::k_fused_tickets<A, MODE, LDSW, MOVES>), g, b, p.lds, e->stream, R, P, t0, n, \
                      tk, p.tab_stride, p.fixed ? 1 : 0, p.pair ? 1 : 0)
-    if (p.fast && p.hybrid)
-      CRL_LAUNCH_TICKETS(true, true, false);
+    if (p.rich && p.moves)
+      CRL_LAUNCH_TICKETS(2, false, true);
+    else if (p.rich)
+      CRL_LAUNCH_TICKETS(2, false, false);
+    else if (p.fast && p.hybrid)
+      CRL_LAUNCH_TICKETS(1, true, false);
     else if (p.fast && p.moves)
-      CRL_LAUNCH_TICKETS(true, false, true);
+      CRL_LAUNCH_TICKETS(1, false, true);
     else if (p.fast)
-      CRL_LAUNCH_TICKETS(true, false, false);
+      CRL_LAUNCH_TICKETS(1, false, false);
     else if (p.hybrid)
-      CRL_LAUNCH_TICKETS(false, true, false);
+      CRL_LAUNCH_TICKETS(0, true, false);
     else
-      CRL_LAUNCH_TICKETS(false, false, false);
+      CRL_LAUNCH_TICKETS(0, false, false);
 #undef CRL_LAUNCH_TICKETS
     return;
   }
@@ -935,12 +945,14 @@ int crl_run_fused(crl_engine* e, int32_t n_steps) {
       if (e->ticket.ensure(3) != hipSuccess) return fail(CRL_E_ALLOC, "ticket counter allocation failed");
       if (!e->hybrid_opt_in) {
         const void* fns[] = {
-            reinterpret_cast<const void*>(&crl::k_fused_tickets<4, true, true, false>),
-            reinterpret_cast<const void*>(&crl::k_fused_tickets<4, false, true, false>),
-            reinterpret_cast<const void*>(&crl::k_fused_tickets<4, true, false, true>),
-            reinterpret_cast<const void*>(&crl::k_fused_tickets<8, true, true, false>),
-            reinterpret_cast<const void*>(&crl::k_fused_tickets<8, false, true, false>),
-            reinterpret_cast<const void*>(&crl::k_fused_tickets<8, true, false, true>)};
+            reinterpret_cast<const void*>(&crl::k_fused_tickets<4, 1, true, false>),
+            reinterpret_cast<const void*>(&crl::k_fused_tickets<4, 0, true, false>),
+            reinterpret_cast<const void*>(&crl::k_fused_tickets<4, 1, false, true>),
+            reinterpret_cast<const void*>(&crl::k_fused_tickets<4, 2, false, true>),
+            reinterpret_cast<const void*>(&crl::k_fused_tickets<8, 1, true, false>),
+            reinterpret_cast<const void*>(&crl::k_fused_tickets<8, 0, true, false>),
+            reinterpret_cast<const void*>(&crl::k_fused_tickets<8, 1, false, true>),
+            reinterpret_cast<const void*>(&crl::k_fused_tickets<8, 2, false, true>)};
         for (const void* fn : fns)
           HIP_TRY(hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, (int)kLdsPerWorkgroup));
         e->hybrid_opt_in = true;

@@ -558,7 +558,7 @@ __device__ __forceinline__ void stage_words(const uint32_t* __restrict__ src, co
   for (int i = i0 + lane; i < total; i += 64) put(i, __builtin_nontemporal_load(src + i));
 }
 
-template <int A, bool FAST, bool LDSW, bool MOVES>
+template <int A, int MODE, bool LDSW, bool MOVES>
 __global__ __launch_bounds__(LDSW ? 320 : 256) void k_fused_tickets(const Rules R, const Ptrs P,
                                                                      const uint64_t t0,
                                                                      const int n_steps,
@@ -566,6 +566,8 @@ __global__ __launch_bounds__(LDSW ? 320 : 256) void k_fused_tickets(const Rules 
                                                                      const int tab_stride,
                                                                      const int fixed_tickets,
                                                                      const int pair_tables) {
+  constexpr bool FAST = MODE >= 1;  // the folded loop ...
+  constexpr bool RICH = MODE == 2;  // ... in its variant with per-cell rewards and per-episode epsilon
   extern __shared__ uint32_t lds[];
   const int n_waves = (int)(blockDim.x >> 6);  // with LDSW the last one works on LDS tables
   const int lane = threadIdx.x & 63;
@@ -623,16 +625,17 @@ __global__ __launch_bounds__(LDSW ? 320 : 256) void k_fused_tickets(const Rules 
         if (l < n_here) {
           const GlobalTable<A> tab{P.Q + (size_t)(env0 + l) * table};
           if (n_steps >= kTouchMinSteps) tab.touch((int)table);
-          run_env_fast<A, true, false>(R, P, env0 + l, t0, n_steps, MovesLds<A>{my_words + l, kTicketEnvs},
-                                       nullptr, tab);
+          run_env_fast<A, true, RICH>(R, P, env0 + l, t0, n_steps, MovesLds<A>{my_words + l, kTicketEnvs},
+                                      RICH && P.cell_reward ? P.cell_reward + (size_t)(env0 + l) * P.S : nullptr,
+                                      tab);
         }
       } else if (live) {
         const GlobalTable<A> tab{P.Q + (size_t)env * table};
         if (n_steps >= kTouchMinSteps) tab.touch((int)table);
         if (kTableMoves)
-          run_env_fast<A, false, false>(R, P, env, t0, n_steps, MovesLds<A>{my_words + lane, 64}, nullptr, tab);
+          run_env_fast<A, false, RICH>(R, P, env, t0, n_steps, MovesLds<A>{my_words + lane, 64}, RICH ? cr : nullptr, tab);
         else if (FAST)
-          run_env_fast<A, false, false>(R, P, env, t0, n_steps, MovesFromMap<A>{my_words + lane, R.W, R.H}, nullptr, tab);
+          run_env_fast<A, false, RICH>(R, P, env, t0, n_steps, MovesFromMap<A>{my_words + lane, R.W, R.H}, RICH ? cr : nullptr, tab);
         else
           run_env_steps<A>(R, P, env, t0, n_steps, MovesFromMap<A>{my_words + lane, R.W, R.H},
                            P.map + (size_t)env * P.map_words, cr, tab);
@@ -671,7 +674,9 @@ __global__ __launch_bounds__(LDSW ? 320 : 256) void k_fused_tickets(const Rules 
         const int l = lane & (kTicketEnvs - 1);
         if (l < n_here) {
           const LdsTable<A> tab{tabs + l * tab_stride};
-          run_env_fast<A, true, false>(R, P, env0 + l, t0, n_steps, MovesLds<A>{my_words + l, kTicketEnvs}, nullptr, tab);
+          run_env_fast<A, true, RICH>(R, P, env0 + l, t0, n_steps, MovesLds<A>{my_words + l, kTicketEnvs},
+                                      RICH && P.cell_reward ? P.cell_reward + (size_t)(env0 + l) * P.S : nullptr,
+                                      tab);
         }
       } else if (live) {
         const LdsTable<A> tab{tabs + lane * tab_stride};

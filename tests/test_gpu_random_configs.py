@@ -53,6 +53,49 @@ def test_random_configs_folded_loop(gpu, oracle, seed):
         assert same(q, st, Q, ost), (seed, case, name, A, W, H, N, T, steps, t0, eps, variant, resident)
 
 
+@pytest.mark.parametrize("seed", [8, 9])
+def test_random_configs_folded_loop_cell_rewards_and_schedules(gpu, oracle, seed):
+    """Per-env maps small enough for LDS with per-cell rewards and / or an epsilon
+    that follows the episode count: the ticket kernel runs the folded loop's variant
+    for them (plain workers only; staged or derived move codes, two lanes per env
+    on small batches)."""
+    rng = np.random.default_rng(seed)
+    for case in range(40):
+        A = int(rng.choice([4, 8]))
+        W, H = (int(rng.integers(2, 40)) for _ in range(2))
+        N = int(rng.choice([1, 31, 33, 64, 65, 500, 2049, 4100, 17000]))
+        T = int(rng.choice([0, 1, 2, 7, 50, 300]))
+        steps, t0 = int(rng.integers(1, 450)), int(rng.integers(0, 5))
+        eps_mode, span = int(rng.choice([0, 2, 3])), int(rng.integers(1, 30))
+        flags = int(rng.choice([0, gpu.REWARD_CELLS, gpu.REWARD_CELLS | gpu.REWARD_BASE_CELLS]))
+        if eps_mode == 0 and flags == 0:
+            flags = gpu.REWARD_CELLS
+        resident = int(rng.choice([0, 64, 200, 1000, 5000]))
+        map_seed = int(rng.integers(0, 1 << 30))
+        if flags:
+            cls, start, cr = gpu.gen_maps_noise(map_seed, N, W, H, 8, 0.2, 0.3, 5.0)
+        else:
+            cls, start = gpu.gen_maps_bernoulli(map_seed, N, N, W, H, 0.15, 0.05)
+            cr = None
+        cfg = gpu.make_config(N, W, H, n_actions=A, episode_len=T, lr=0.2, gamma=0.9, reward_flags=flags,
+                              eps_mode=eps_mode, eps0=float(rng.choice([0.0, 0.3, 0.6, 1.0])), eps_decay=0.9,
+                              eps_end=0.05, eps_span=span, seed=map_seed, trap_reward=-0.5)
+        with gpu.Engine(cfg, 0) as eng:
+            eng.set_maps(cls, start, cr)
+            eng.set_resident_envs(resident)
+            eng.step_count = t0
+            name = eng.fused_kernel_info()["name"]
+            third = steps // 3
+            for c in (third, steps - 2 * third, third):
+                eng.run_fused(c)
+            q, st = eng.q_get(0, N), eng.get_state()
+        Q = np.zeros((N, W * H, A), np.float32)
+        ost = oracle.new_state(cfg, start)
+        oracle.run(cfg, cls, cr, start, Q, ost, t0, steps)
+        assert name.startswith("k_fused_tickets") and "fast+" in name, name
+        assert same(q, st, Q, ost), (seed, case, name, A, W, H, N, T, steps, t0, eps_mode, flags, resident)
+
+
 @pytest.mark.parametrize("seed", [4, 5])
 def test_random_configs_folded_loop_large_or_shared_maps(gpu, oracle, seed):
     """The folded loop's variant for maps that are shared or too large for LDS:
