@@ -531,10 +531,14 @@ __global__ __launch_bounds__(256) void k_fused_per_env(const Rules R, const Ptrs
 // split between the two kinds follows their speed; which worker steps an env does
 // not change its results.
 //
-// FAST selects the folded loop (run_env_fast), which works on move codes: the
-// LDS wave always stages the pre-built codes of its envs; the table waves stage
-// them too with MOVES, and otherwise stage the (four times smaller) class maps
-// and derive the codes while their row loads are in flight.
+// MODE 0 is the general loop; 1 and 2 select the folded loop (run_env_fast; 2: its
+// variant with per-cell rewards and per-episode epsilon), which works on move
+// codes: the LDS wave always stages the pre-built codes of its envs; the table
+// waves stage them too with MOVES, and otherwise stage the (four times smaller)
+// class maps and derive the codes while their row loads are in flight.  With
+// staged codes and `pair_tables` a table wave takes one ticket instead of two and
+// gives every env two lanes, like the LDS wave: for batches too small to fill the
+// chip with 64-env waves.
 constexpr int kTicketEnvs = 32;
 
 // `count` envs' words (`wpe` per env, contiguous in HBM) into [word][lane]; eight
