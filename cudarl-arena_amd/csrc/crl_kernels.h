@@ -363,19 +363,21 @@ __device__ __forceinline__ void run_env_fast(const Rules& R, const Ptrs& P, cons
   // own block, and (PAIR) the partner lane's: {blk, nxt} = the next two blocks
   auto two_blocks = [&](uint64_t b, Philox4& first, Philox4& second) {
     const Philox4 own = explore_block(R.seed, (uint32_t)env, b + (upper ? 1 : 0));
-    Philox4 other;
-    other.w0 = (uint32_t)__shfl((int)own.w0, lane ^ 32);
-    other.w1 = (uint32_t)__shfl((int)own.w1, lane ^ 32);
-    other.w2 = (uint32_t)__shfl((int)own.w2, lane ^ 32);
-    other.w3 = (uint32_t)__shfl((int)own.w3, lane ^ 32);
-    first.w0 = upper ? other.w0 : own.w0;
-    first.w1 = upper ? other.w1 : own.w1;
-    first.w2 = upper ? other.w2 : own.w2;
-    first.w3 = upper ? other.w3 : own.w3;
-    second.w0 = upper ? own.w0 : other.w0;
-    second.w1 = upper ? own.w1 : other.w1;
-    second.w2 = upper ? own.w2 : other.w2;
-    second.w3 = upper ? own.w3 : other.w3;
+    // v_permlane32_swap exchanges the upper 32 lanes of its first operand with the
+    // lower 32 of its second: given the same value twice it returns the lower
+    // half's words in both halves (block b) and the upper half's (block b + 1)
+    const auto w0 = __builtin_amdgcn_permlane32_swap(own.w0, own.w0, false, false);
+    const auto w1 = __builtin_amdgcn_permlane32_swap(own.w1, own.w1, false, false);
+    const auto w2 = __builtin_amdgcn_permlane32_swap(own.w2, own.w2, false, false);
+    const auto w3 = __builtin_amdgcn_permlane32_swap(own.w3, own.w3, false, false);
+    first.w0 = w0[0];
+    first.w1 = w1[0];
+    first.w2 = w2[0];
+    first.w3 = w3[0];
+    second.w0 = w0[1];
+    second.w1 = w1[1];
+    second.w2 = w2[1];
+    second.w3 = w3[1];
   };
   Philox4 blk, nxt{};
   bool have_nxt = PAIR;
