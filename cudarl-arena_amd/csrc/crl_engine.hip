@@ -367,7 +367,8 @@ void launch_fused_a(const crl_engine* e, const FusedPlan& p, uint64_t t0, int n)
   const crl::Rules R = e->rules();
   const crl::Ptrs P = e->ptrs();
   if (p.tickets) {
-    hipLaunchKernelGGL(crl::k_fill_u32, dim3(1), dim3(64), 0, e->stream, e->ticket.p, 0u, 3);
+    // (tickets dealt by position use no counter; the kernel itself notes who did how much)
+    if (!p.fixed) hipLaunchKernelGGL(crl::k_fill_u32, dim3(1), dim3(64), 0, e->stream, e->ticket.p, 0u, 3);
     const dim3 g(p.grid), b(p.block);
     unsigned* tk = e->ticket.p;
 #define CRL_LAUNCH_TICKETS(MODE, LDSW, MOVES)                                                       \
