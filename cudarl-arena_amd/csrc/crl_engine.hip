@@ -257,15 +257,15 @@ FusedPlan plan_fused(const crl_engine* e, int n_steps) {
     // runs with every env in flight)
     if ((size_t)e->N * table_bytes > kTableBytesInFlight && n_steps >= kInFlightMinSteps)
       resident = std::max<long>(kMinEnvsInFlight, (long)(kTableBytesInFlight / table_bytes));
-    // The batch passes through in rounds of that many envs; a last round that fills
-    // a fraction of the chip costs a whole one.  Even the rounds out, in whole waves
-    // per compute unit (65,536 envs with 32x32 maps: 3.5e10 env-steps/s as one round
-    // of 49,152 and one of 16,384, 4.4e10 as two of 32,768).
+    // The batch goes through the chip in shifts of that many envs; a last shift that
+    // fills a fraction of the chip costs a whole one.  Even the shifts out, in whole
+    // waves per compute unit (65,536 envs with 32x32 maps: 3.5e10 env-steps/s as one
+    // shift of 49,152 and one of 16,384, 4.4e10 as two of 32,768).
     if (resident < e->N) {
-      const long rounds = (e->N + resident - 1) / resident;
-      const long per_round = (e->N + rounds - 1) / rounds;
+      const long shifts = (e->N + resident - 1) / resident;
+      const long per_shift = (e->N + shifts - 1) / shifts;
       const long unit = 64L * kComputeUnits;
-      resident = std::min(resident, (per_round + unit - 1) / unit * unit);
+      resident = std::min(resident, (per_shift + unit - 1) / unit * unit);
     }
   }
   p.tickets = p.map_kind == 0;
