@@ -3,21 +3,27 @@
 
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload c4|c2|c3|c5]
 
-One "step" advances every env of the workload by one select -> step -> update.
-W warm-up steps run first, then exactly K steps are timed with the inputs (maps,
-tables, state) already resident in HBM.  Prints ONE JSON line.
+One "step" of this benchmark is ONE PASS OF THE WORKLOAD: every env of the
+configuration advanced by the configuration's own number of env-steps (c4: 1000
+select -> step -> update rounds for each of 1,048,576 envs, one kernel launch).
+W warm-up passes run first, then exactly K passes are timed with the inputs
+(maps, tables, state) already resident in HBM; the launch length never depends
+on K.  Prints ONE JSON line.
 
 Workloads (the benchmark configurations, numbered from 1):
-  c2  4096 envs, 32x32, per-env tables (64 MB; cache resident)
-  c3  65536 envs sharing one 64x64 map and ONE table (ordered reduction per step)
-  c4  1,048,576 envs, 16x16, per-env tables (4 GB; the HBM-bound config)  [default]
-  c5  8192 envs, 256x256, 8 actions, per-env tables (16 GB)
+  c2  4096 envs, 32x32, per-env tables (64 MB; cache resident), 10,000 env-steps per pass
+  c3  65536 envs sharing one 64x64 map and ONE table (ordered reduction per step), 1000 per pass
+  c4  1,048,576 envs, 16x16, per-env tables (4 GB; the HBM-bound config), 1000 per pass  [default]
+  c5  8192 envs, 256x256, 8 actions, per-env tables (16 GB), 1024 per pass
 """
 import argparse
 import ctypes as C
 import json
 import os
+import statistics
+import subprocess
 import sys
+import tempfile
 import threading
 import time
 
@@ -30,18 +36,26 @@ import pycrl  # noqa: E402
 HBM_PEAK_GBS = 8000.0  # MI355X HBM3E
 
 WORKLOADS = {
-    # algorithmic bytes per env-step: 22 B of state/outputs + (4A+4) B of table
+    # bytes: algorithmic bytes per env-step = 22 B of state/outputs + (4A+4) B of table
     # traffic (one new row, one write) + S/(8T) B of map per episode (+4 B/cell reward)
-    "c2": dict(n=4096, w=32, h=32, a=4, t=256, steps=10000, warmup=256, bytes=42.5,
-               name="c2: 4096 envs 32x32, per-env tables 1024x4, eps 0.1, T=256"),
-    "c3": dict(n=65536, w=64, h=64, a=4, t=0, steps=1000, warmup=50, bytes=24.0,
-               name="c3: 65536 envs, shared 64x64 map, one shared table 4096x4, ordered reduction"),
+    # launch_steps: env-steps every env takes in one pass (the configuration's own length)
+    "c2": dict(n=4096, launch_steps=10000, bytes=42.5,
+               name="c2: 4096 envs 32x32, per-env tables 1024x4, eps 0.1, T=256, 10000 steps"),
+    "c3": dict(n=65536, launch_steps=1000, bytes=24.0,
+               name="c3: 65536 envs, shared 64x64 map, one shared table 4096x4, ordered reduction, "
+                    "lr 0.05 (as specified: the table overflows within ~100 steps), 1000 steps"),
+    # the same with a step size small enough for the table to stay finite, so that the
+    # reduction is timed on keys spread over the map instead of piled up behind NaN rows
+    "c3f": dict(n=65536, launch_steps=1000, bytes=24.0,
+                name="c3 with lr 0.0005 (finite table): 65536 envs, shared 64x64 map, one shared "
+                     "table 4096x4, ordered reduction, 1000 steps"),
     # traffic: HBM bytes per env-step from rocprofv3 FETCH_SIZE x2.000 + WRITE_SIZE x1.000
     # (profiles/k_fused_tickets_c4.md), valid for the default launch only
-    "c4": dict(n=1 << 20, w=16, h=16, a=4, t=128, steps=1000, warmup=128, bytes=42.25, traffic=30.8,
-               name="c4: 1048576 envs 16x16, per-env tables 256x4 (4 GB), traps, eps 0.1, T=128"),
-    "c5": dict(n=8192, w=256, h=256, a=8, t=1024, steps=1024, warmup=64, bytes=70.0,
-               name="c5: 8192 envs 256x256, 8 actions, per-env tables 65536x8 (16 GB), cell rewards"),
+    "c4": dict(n=1 << 20, launch_steps=1000, bytes=42.25, traffic=30.8,
+               name="c4: 1048576 envs 16x16, per-env tables 256x4 (4 GB), traps, eps 0.1, T=128, 1000 steps"),
+    "c5": dict(n=8192, launch_steps=1024, bytes=70.0, traffic=None,
+               name="c5: 8192 envs 256x256, 8 actions, per-env tables 65536x8 (16 GB), cell rewards, "
+                    "eps 1.0->0.05 over 100 episodes, T=1024, 1024 steps"),
 }
 
 
@@ -52,9 +66,9 @@ def build_workload(key, n_override=None):
         cfg = pycrl.make_config(n, 32, 32, episode_len=256, lr=0.1, gamma=0.99, eps0=0.1, seed=0)
         cls, start = pycrl.gen_maps_bernoulli(0, n, n, 32, 32, 0.2)
         return cfg, cls, start, None
-    if key == "c3":
+    if key in ("c3", "c3f"):
         cfg = pycrl.make_config(n, 64, 64, table_mode=pycrl.TABLE_SHARED, map_mode=pycrl.MAP_SHARED,
-                                lr=0.05, gamma=0.99, eps0=0.2, seed=0)
+                                lr=0.05 if key == "c3" else 0.0005, gamma=0.99, eps0=0.2, seed=0)
         cls, start = pycrl.gen_maps_bernoulli(0, 1, n, 64, 64, 0.15)
         return cfg, cls, start, None
     if key == "c4":
@@ -82,10 +96,10 @@ class HipEvents:
         self.hip.hipEventElapsedTime.argtypes = [C.POINTER(C.c_float), C.c_void_p, C.c_void_p]
         self.hip.hipEventDestroy.argtypes = [C.c_void_p]
 
-    def pair(self):
-        a, b = C.c_void_p(), C.c_void_p()
-        assert self.hip.hipEventCreate(C.byref(a)) == 0 and self.hip.hipEventCreate(C.byref(b)) == 0
-        return a, b
+    def new(self):
+        a = C.c_void_p()
+        assert self.hip.hipEventCreate(C.byref(a)) == 0
+        return a
 
     def record(self, ev):
         assert self.hip.hipEventRecord(ev, None) == 0
@@ -96,10 +110,16 @@ class HipEvents:
         assert self.hip.hipEventElapsedTime(C.byref(ms), a, b) == 0
         return float(ms.value)
 
+    def free(self, evs):
+        for e in evs:
+            self.hip.hipEventDestroy(e)
 
-def time_gpu(key, steps, warmup, launches=1, n_override=None, resident=0, variant=0):
-    """-> dict(steps_per_s, ms_per_step, kernel_ms, wall_s, info)"""
+
+def time_gpu(key, reps, warm_reps, launch_steps=None, n_override=None, resident=0, variant=0):
+    """`reps` timed passes of `launch_steps` env-steps per env (default: the
+    workload's own length) after `warm_reps` untimed ones."""
     wl = WORKLOADS[key]
+    per = launch_steps or wl["launch_steps"]
     cfg, cls, start, cr = build_workload(key, n_override)
     n = cfg.n_envs
     ev = HipEvents()
@@ -110,49 +130,76 @@ def time_gpu(key, steps, warmup, launches=1, n_override=None, resident=0, varian
             eng.set_resident_envs(resident)
         if variant:
             eng.set_fused_variant(variant)
-        info = eng.fused_kernel_info()
-        if warmup:
-            eng.run_fused(warmup)
+        info = eng.fused_kernel_info(per)
+        for _ in range(warm_reps):
+            eng.run_fused(per)
         eng.sync()
-        a, b = ev.pair()
-        per_launch = steps // launches
-        counts = [per_launch] * launches
-        counts[-1] += steps - per_launch * launches
+        marks = [ev.new() for _ in range(reps + 1)]
         t0 = time.perf_counter()
-        ev.record(a)
-        for c in counts:
-            eng.run_fused(c)
-        ev.record(b)
+        ev.record(marks[0])
+        for i in range(reps):
+            eng.run_fused(per)
+            ev.record(marks[i + 1])
         eng.sync()
         wall = time.perf_counter() - t0
-        dev_ms = ev.elapsed_ms(a, b)
+        rep_ms = [ev.elapsed_ms(marks[i], marks[i + 1]) for i in range(reps)]
+        ev.free(marks)
         st = eng.get_state()
         split = eng.fused_split()
+        q_probe = eng.q_get(0)
+    dev_ms = sum(rep_ms)
     secs = max(wall, dev_ms * 1e-3)
-    return dict(n=n, steps_per_s=n * steps / secs, ms_per_step=secs * 1e3 / steps, device_ms=dev_ms,
-                wall_s=wall, launches=launches, info=info, split=split, episodes_min=int(st["episode"].min()),
-                bytes_per_step=wl["bytes"])
+    return dict(n=n, launch_steps=per, reps=reps, env_steps=n * per * reps, steps_per_s=n * per * reps / secs,
+                ms_per_rep=secs * 1e3 / reps, device_ms=dev_ms, rep_ms=rep_ms, wall_s=wall, info=info,
+                split=split, episodes_min=int(st["episode"].min()), bytes_per_step=wl["bytes"],
+                table_finite=bool(np.isfinite(q_probe).all()))
 
 
-def time_cpu(key, n_sample, steps, threads):
-    """The oracle (a scalar C port of the reference's kernels) on `threads` host
-    threads over the first n_sample envs of the same workload."""
+def _cpu_model():
+    try:
+        with open("/proc/cpuinfo") as f:
+            for line in f:
+                if line.lower().startswith("model name"):
+                    return line.split(":", 1)[1].strip()
+    except OSError:
+        pass
+    return "unknown"
+
+
+def _native_oracle():
+    """The oracle compiled for this host (-O3 -march=native, contraction still off:
+    same results), for the timing leg only; falls back to the library the tests use."""
     sys.path.insert(0, os.path.join(ROOT, "tests"))
     from conftest import ORACLE_SO, Oracle
-    if not os.path.exists(ORACLE_SO):
-        import subprocess
-        subprocess.check_call(["make", "-C", os.path.join(ROOT, "oracle"), "-s"])
-    orc = Oracle(C.CDLL(ORACLE_SO))
+    src = os.path.join(ROOT, "oracle", "crl_oracle.c")
+    out = os.path.join(tempfile.mkdtemp(prefix="crl_oracle_"), "libcrl_oracle_native.so")
+    cmd = ["gcc", "-O3", "-march=native", "-fPIC", "-std=c11", "-ffp-contract=off", "-fno-fast-math",
+           "-shared", "-o", out, src, "-lm"]
+    try:
+        subprocess.check_call(cmd, stdout=subprocess.DEVNULL, stderr=subprocess.DEVNULL)
+        return Oracle(C.CDLL(out)), "-O3 -march=native -ffp-contract=off"
+    except (OSError, subprocess.CalledProcessError):
+        if not os.path.exists(ORACLE_SO):
+            subprocess.check_call(["make", "-C", os.path.join(ROOT, "oracle"), "-s"])
+        return Oracle(C.CDLL(ORACLE_SO)), "-O2 -ffp-contract=off"
+
+
+def time_cpu(orc, key, n_sample, steps, threads):
+    """The oracle (a scalar C port of the reference's kernels) on `threads` host
+    threads over the first n_sample envs of the same workload."""
+    from conftest import Oracle
     cfg, cls, start, cr = build_workload(key, n_sample)
     S, A = cfg.width * cfg.height, cfg.n_actions
     st = orc.new_state(cfg, start)
     if cfg.table_mode == pycrl.TABLE_SHARED:
+        # one table, one ordered reduction per step: the port runs it on one thread
         Q = np.zeros((1, S, A), np.float32)
         t0 = time.perf_counter()
         orc.run(cfg, cls, cr, start, Q, st, 0, steps)
         dt = time.perf_counter() - t0
         return n_sample * steps / dt, 1, dt
     Q = np.zeros((n_sample, S, A), np.float32)
+    Q.fill(0.0)  # pages touched before the clock starts
     p = Oracle._p
     bounds = [n_sample * i // threads for i in range(threads + 1)]
 
@@ -172,24 +219,70 @@ def time_cpu(key, n_sample, steps, threads):
     return n_sample * steps / dt, threads, dt
 
 
+def cpu_baseline(key, full_n):
+    """Single-thread and all-threads figures of the CPU port on this host."""
+    orc, flags = _native_oracle()
+    nproc = os.cpu_count() or 1
+    try:
+        usable = len(os.sched_getaffinity(0))
+    except AttributeError:
+        usable = nproc
+    # a shared GPU host gives one job a share of its cores and says so in
+    # OMP_NUM_THREADS; more threads than that would time the neighbours' load
+    share = int(os.environ.get("OMP_NUM_THREADS", "0") or 0)
+    threads = max(1, min(usable, share) if share > 0 else usable)
+    steps = {"c2": 10000, "c3": 1000, "c3f": 1000, "c4": 1000, "c5": 1024}[key]
+    n1 = {"c2": 256, "c3": full_n, "c3f": full_n, "c4": 65536, "c5": 128}[key]
+    v1, _, dt1 = time_cpu(orc, key, min(n1, full_n), steps, 1)
+    out = {"unit": "env-steps/s", "kind": "port", "nproc": nproc, "cpu_model": _cpu_model(),
+           "compiler_flags": "gcc " + flags,
+           "single_thread": {"value": v1, "cores": 1,
+                             "sample": "%d envs x %d steps of the same workload, %.1f s" % (min(n1, full_n), steps, dt1)}}
+    if WORKLOADS[key]["name"].startswith("c3"):
+        out.update(value=v1, cores=1, sample=out["single_thread"]["sample"] +
+                   " (one shared table: the port's ordered reduction is serial)")
+        return out
+    # all threads: the full configuration when that is about 10 s of wall time, else a share of it
+    n_all = int(min(full_n, max(threads * 64, v1 * threads * 10.0 / steps)))
+    va, cores, dta = time_cpu(orc, key, n_all, steps, threads)
+    out.update(value=va, cores=cores,
+               sample="%d of %d envs x %d steps of the same workload, %.1f s wall on %d threads"
+                      % (n_all, full_n, steps, dta, cores))
+    return out
+
+
+def side_figure(key, reps, warm, launch_steps=None):
+    r = time_gpu(key, reps, warm, launch_steps)
+    return {"workload": WORKLOADS[key]["name"], "value": r["steps_per_s"], "unit": "env-steps/s",
+            "n_envs": r["n"], "steps_per_launch": r["launch_steps"], "launches_timed": reps,
+            "us_per_env_step_round": r["device_ms"] * 1e3 / (reps * r["launch_steps"]),
+            "median_launch_ms": statistics.median(r["rep_ms"]), "kernel": r["info"]["name"],
+            "roofline_frac": r["n"] * r["launch_steps"] * reps * r["bytes_per_step"] / (r["device_ms"] * 1e-3) / 1e9
+                             / HBM_PEAK_GBS,
+            "table_finite_at_end": r["table_finite"]}
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=None)
-    ap.add_argument("--warmup", type=int, default=None)
+    ap.add_argument("--steps", type=int, default=20, help="timed passes of the workload (one launch each)")
+    ap.add_argument("--warmup", type=int, default=3, help="untimed passes before them")
     ap.add_argument("--workload", default="c4", choices=sorted(WORKLOADS))
-    ap.add_argument("--launches", type=int, default=1, help="split the K timed steps over this many launches")
+    ap.add_argument("--launch-steps", type=int, default=None,
+                    help="env-steps per launch instead of the workload's own (not a headline figure)")
     ap.add_argument("--envs", type=int, default=None, help="override the env count (not a headline figure)")
     ap.add_argument("--resident", type=int, default=0, help="envs in flight at once (0 = automatic)")
     ap.add_argument("--variant", type=int, default=0, help="fused kernel: 0 automatic, 1 plain, 2 hybrid")
     ap.add_argument("--probe-copy", type=int, default=0, metavar="MIB",
                     help="only run one plain copy kernel of this many MiB (calibrates rocprofv3 counters)")
     ap.add_argument("--no-cpu", action="store_true", help="skip the cpu_baseline leg")
-    ap.add_argument("--no-also", action="store_true", help="skip the short c2/c3/c5 side measurements")
+    ap.add_argument("--no-also", action="store_true", help="skip the side measurements of the other configs")
     args = ap.parse_args()
     if args.gpus != 1:
         raise SystemExit("bench.py: this build runs on ONE GPU (envs shard trivially, but no second "
                          "GPU is used in this run); got --gpus %d" % args.gpus)
+    if args.steps < 1 or args.warmup < 0:
+        raise SystemExit("bench.py: --steps must be at least 1 and --warmup non-negative")
     lib = pycrl.load()
     if lib.crl_device_count() < 1:
         raise SystemExit("bench.py: no HIP device: %s" % lib.crl_last_error().decode())
@@ -200,58 +293,58 @@ def main():
         return
     key = args.workload
     wl = WORKLOADS[key]
-    steps = args.steps if args.steps is not None else wl["steps"]
-    warmup = args.warmup if args.warmup is not None else wl["warmup"]
-    g = time_gpu(key, steps, warmup, args.launches, args.envs, args.resident, args.variant)
+    g = time_gpu(key, args.steps, args.warmup, args.launch_steps, args.envs, args.resident, args.variant)
 
-    achieved = g["steps_per_s"] * wl["bytes"] / 1e9
-    # the dominant kernel's own duration (device events around its launches)
-    kern_achieved = g["n"] * steps * wl["bytes"] / (g["device_ms"] * 1e-3) / 1e9
+    per_launch_units = g["n"] * g["launch_steps"]
+    bytes_per_launch = per_launch_units * wl["bytes"]
+    avg_launch_ms = g["device_ms"] / g["reps"]
+    achieved = bytes_per_launch / (avg_launch_ms * 1e-3) / 1e9  # the dominant kernel, HIP events around its launches
+    default_shape = (not args.launch_steps and not args.envs and not args.resident and not args.variant)
     out = {
         "metric": "env-steps/sec (step+select+TD update) at 1 MI355X",
         "value": g["steps_per_s"],
         "unit": "env-steps/s",
         "n_gpus": 1,
-        "steps": steps,
-        "warmup": warmup,
-        "ms_per_step": g["ms_per_step"],
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": g["ms_per_rep"],
         "higher_is_better": True,
         "scaling": "weak",
         "vs_baseline": None,
         "dtype": "f32",
-        "data": "synthetic (Philox-seeded maps, zero-initialised tables)",
-        "config": {"workload": wl["name"], "n_envs": g["n"], "steps_per_launch": steps // args.launches,
+        "data": "synthetic (Philox-seeded maps, zero-initialised tables, trained on by the warm-up passes)",
+        "config": {"workload": wl["name"], "n_envs": g["n"], "steps_per_launch": g["launch_steps"],
+                   "one_bench_step": "one launch = %d env-steps for each of %d envs" % (g["launch_steps"], g["n"]),
+                   "launches_timed": g["reps"], "env_steps_timed": g["env_steps"],
+                   "timed_region_ms": g["wall_s"] * 1e3,
+                   "launch_ms_median": statistics.median(g["rep_ms"]), "launch_ms_min": min(g["rep_ms"]),
+                   "launch_ms_max": max(g["rep_ms"]),
+                   "value_at_median_launch": per_launch_units / (statistics.median(g["rep_ms"]) * 1e-3),
                    "kernel": g["info"]["name"], "grid": g["info"]["grid"], "block": g["info"]["block"],
                    "lds_bytes": g["info"]["lds_bytes"],
                    "envs_stepped_from_hbm_tables": g["split"][0], "envs_stepped_from_lds_tables": g["split"][1]},
-        "roofline": {"bound": "hbm", "achieved": kern_achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                     "frac": kern_achieved / HBM_PEAK_GBS, "traffic": None,
+        "roofline": {"bound": "hbm", "achieved": achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                     "frac": achieved / HBM_PEAK_GBS, "traffic": None,
                      "algorithmic_bytes_per_env_step": wl["bytes"],
-                     "kernel_ms_per_launch": g["device_ms"] / args.launches,
-                     "whole_job_GBps": achieved},
+                     "algorithmic_bytes_per_launch": bytes_per_launch,
+                     "kernel_ms_per_launch": avg_launch_ms},
     }
-    if ("traffic" in wl and steps == wl["steps"] and args.launches == 1 and not args.envs
-            and not args.resident):
-        # measured in separate rocprofv3 --pmc runs of this same command, not in this run
-        out["roofline"]["traffic"] = wl["traffic"] * g["n"] * steps
+    if wl.get("traffic") and default_shape:
+        # bytes past the L2 per launch, measured in separate rocprofv3 --pmc runs of this
+        # same command (profiles/), not in this run
+        out["roofline"]["traffic"] = wl["traffic"] * per_launch_units
 
     if not args.no_cpu:
-        threads = min(16, os.cpu_count() or 1)
-        # about 10-30 s of CPU work each (the wall time is that divided by the threads)
-        n_sample = {"c2": 4096, "c3": 65536, "c4": 1 << 18, "c5": 2048}[key]
-        cpu_steps = {"c2": 50000, "c3": 1500, "c4": 1000, "c5": 16384}[key]
-        v, cores, dt = time_cpu(key, min(n_sample, g["n"]), cpu_steps, threads)
-        out["cpu_baseline"] = {"value": v, "unit": "env-steps/s", "cores": cores, "kind": "port",
-                               "sample": "%d envs x %d steps of the same workload, %.1f s wall on %d threads"
-                                         % (min(n_sample, g["n"]), cpu_steps, dt, cores)}
+        out["cpu_baseline"] = cpu_baseline(key, g["n"])
     if not args.no_also and not args.envs:
         also = {}
-        for k2, s2, w2 in (("c3", 300, 20), ("c2", 4000, 256), ("c5", 1024, 64)):
-            if k2 == key:
-                continue
-            r = time_gpu(k2, s2, w2)
-            also[k2] = {"workload": WORKLOADS[k2]["name"], "value": r["steps_per_s"], "unit": "env-steps/s",
-                        "steps": s2, "ms_per_step": r["ms_per_step"], "kernel": r["info"]["name"]}
+        for k2, reps, warm in (("c3", 3, 1), ("c3f", 3, 1), ("c2", 5, 1), ("c5", 5, 1)):
+            if k2 != key:
+                also[k2] = side_figure(k2, reps, warm)
+        if key == "c4" and default_shape:
+            # what a caller that asks for a few steps at a time gets: another launch plan
+            # (every env in flight, class maps staged, tables never in LDS)
+            also["c4_20_steps_per_launch"] = side_figure("c4", 20, 5, 20)
         out["also"] = also
     print(json.dumps(out))
 

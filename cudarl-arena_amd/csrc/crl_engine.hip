@@ -8,6 +8,8 @@
 #include <algorithm>
 #include <cstdlib>
 #include <cstring>
+#include <exception>
+#include <memory>
 #include <new>
 #include <string>
 #include <vector>
@@ -37,6 +39,21 @@ int fail(int code, const char* fmt, ...) {
       return fail(_e == hipErrorOutOfMemory ? CRL_E_ALLOC : CRL_E_DEVICE, "%s: %s (%s:%d)", \
                   #expr, hipGetErrorString(_e), __FILE__, __LINE__);                    \
   } while (0)
+
+// Runs the body of an entry point that allocates host memory or starts threads:
+// nothing may throw across the C ABI.
+template <class F>
+int guarded(F&& body) {
+  try {
+    return body();
+  } catch (const std::bad_alloc&) {
+    return fail(CRL_E_ALLOC, "host allocation failed");
+  } catch (const std::exception& x) {
+    return fail(CRL_E_DEVICE, "%s", x.what());
+  } catch (...) {
+    return fail(CRL_E_DEVICE, "unknown failure");
+  }
+}
 
 template <class T>
 struct DevBuf {
@@ -118,6 +135,7 @@ struct crl_engine {
   // host mirrors for crl_set_cell
   std::vector<uint8_t> h_class;
   std::vector<float> h_cell_reward;
+  uint32_t stage_word = 0;  // source of crl_set_cell's asynchronous one-word copy
 
   crl::Rules rules() const {
     crl::Rules R{};
@@ -313,19 +331,24 @@ FusedPlan plan_fused(const crl_engine* e, int n_steps) {
       p.block = 64 * ((int)hbm_waves + 1);
       p.lds = hbm_waves * map_lds + lds_wave + tables_lds;
     } else {
-      long waves = 4;
+      long waves = 4, workers;  // waves per workgroup, 64-env workers in flight
       if (tickets / 2 < 4 * kComputeUnits) {
         // fewer 64-env workers than SIMDs on the chip: one-wave workgroups spread
         // them over the compute units instead of packing four per unit
         waves = 1;
-        p.grid = (int)std::min<long>(std::max<long>(1, resident / 64), (tickets + 1) / 2);
+        workers = std::min<long>(std::max<long>(1, resident / 64), (tickets + 1) / 2);
       } else if (resident <= 4L * 64 * kComputeUnits) {
         // at most four waves per compute unit: spread them over all units
         waves = std::max<long>(1, resident / (64L * kComputeUnits));
-        p.grid = (int)std::min<long>(kComputeUnits, (tickets + 2 * waves - 1) / (2 * waves));
+        workers = waves * std::min<long>(kComputeUnits, (tickets + 2 * waves - 1) / (2 * waves));
       } else {
-        p.grid = (int)std::min<long>(std::max<long>(1, resident / 256), (tickets + 7) / 8);
+        workers = 4 * std::min<long>(std::max<long>(1, resident / 256), (tickets + 7) / 8);
       }
+      // every wave stages the maps of its 64 envs in its own LDS slice: large maps
+      // leave room for fewer waves per workgroup (one always fits: map_kind 0
+      // means 64 maps take at most 64 KB), the workers in flight stay the same
+      while (waves > 1 && (size_t)waves * map_lds > kLdsPerWorkgroup) --waves;
+      p.grid = (int)((workers + waves - 1) / waves);
       p.block = 64 * (int)waves;
       // staging the codes (four times the class map) pays off over a long launch only:
       // 1M envs of config 4, one step per launch 7.7e9 -> 1.4e10 with class maps, 48 steps 3.6e10 -> 3.7e10
@@ -537,6 +560,22 @@ int shared_step(crl_engine* e, uint64_t t, int trace_row) {
   return CRL_OK;
 }
 
+// sizes that follow from the configuration alone
+void set_geometry(crl_engine* e, const crl_config& cfg) {
+  e->cfg = cfg;
+  e->N = cfg.n_envs;
+  e->W = cfg.width;
+  e->H = cfg.height;
+  e->A = cfg.n_actions;
+  e->S = (size_t)cfg.width * cfg.height;
+  e->K = e->S * e->A;
+  e->n_maps = cfg.map_mode == CRL_MAP_SHARED ? 1 : e->N;
+  e->n_tables = cfg.table_mode == CRL_TABLE_SHARED ? 1 : e->N;
+  e->map_words = (int)((e->S + 15) / 16);
+  const size_t cells_per_word = 16 / (size_t)e->A;
+  e->mv_words = (int)((e->S + cells_per_word - 1) / cells_per_word);
+}
+
 int check_engine(const crl_engine* e) {
   if (!e) return fail(CRL_E_ARG, "null engine");
   hipError_t err = hipSetDevice(e->device);
@@ -576,21 +615,7 @@ int upload_maps(crl_engine* e) {
   return CRL_OK;
 }
 
-}  // namespace
-
-extern "C" {
-
-const char* crl_last_error(void) { return g_err.c_str(); }
-const char* crl_version(void) { return CRL_VERSION; }
-
-int crl_device_count(void) {
-  int n = 0;
-  hipError_t e = hipGetDeviceCount(&n);
-  if (e != hipSuccess) return fail(CRL_E_DEVICE, "hipGetDeviceCount: %s", hipGetErrorString(e));
-  return n;
-}
-
-int crl_create(const crl_config* cfg, int device, crl_engine** out) {
+int create_engine(const crl_config* cfg, int device, crl_engine** out) {
   if (!out) return fail(CRL_E_ARG, "out is null");
   *out = nullptr;
   int rc = crl::validate_config(cfg, g_err);
@@ -603,19 +628,10 @@ int crl_create(const crl_config* cfg, int device, crl_engine** out) {
   if (device < 0 || device >= ndev) return fail(CRL_E_ARG, "device %d out of range [0,%d)", device, ndev);
   HIP_TRY(hipSetDevice(device));
 
-  crl_engine* e = new (std::nothrow) crl_engine();
-  if (!e) return fail(CRL_E_ALLOC, "host allocation failed");
-  e->cfg = *cfg;
+  std::unique_ptr<crl_engine> own(new crl_engine());  // freed on every early return and on a throw
+  crl_engine* e = own.get();
+  set_geometry(e, *cfg);
   e->device = device;
-  e->N = cfg->n_envs;
-  e->W = cfg->width;
-  e->H = cfg->height;
-  e->A = cfg->n_actions;
-  e->S = (size_t)cfg->width * cfg->height;
-  e->K = e->S * e->A;
-  e->n_maps = cfg->map_mode == CRL_MAP_SHARED ? 1 : e->N;
-  e->n_tables = cfg->table_mode == CRL_TABLE_SHARED ? 1 : e->N;
-  e->map_words = (int)((e->S + 15) / 16);
 
   const size_t N = (size_t)e->N;
   std::vector<float> eps = crl::build_eps_table(*cfg);
@@ -634,12 +650,7 @@ int crl_create(const crl_config* cfg, int device, crl_engine** out) {
   acc(e->done.alloc(N));
   acc(e->action.alloc(N));
   acc(e->map.alloc((size_t)e->n_maps * e->map_words));
-  // move codes of every map, for the fused loops
-  {
-    const size_t cells_per_word = 16 / (size_t)e->A;
-    e->mv_words = (int)((e->S + cells_per_word - 1) / cells_per_word);
-    acc(e->moves.alloc((size_t)e->n_maps * e->mv_words));
-  }
+  acc(e->moves.alloc((size_t)e->n_maps * e->mv_words));  // move codes of every map, for the fused loops
   if (cells) acc(e->cell_reward.alloc((size_t)e->n_maps * e->S));
   acc(e->Q.alloc((size_t)e->n_tables * e->K));
   acc(e->eps_tab.alloc(eps.size()));
@@ -661,18 +672,15 @@ int crl_create(const crl_config* cfg, int device, crl_engine** out) {
   }
   if (a != hipSuccess) {
     const int code = a == hipErrorOutOfMemory ? CRL_E_ALLOC : CRL_E_DEVICE;
-    delete e;
     return fail(code, "device allocation failed: %s", hipGetErrorString(a));
   }
   try {
     e->h_class.assign((size_t)e->n_maps * e->S, (uint8_t)CRL_CELL_FREE);
     if (cells) e->h_cell_reward.assign((size_t)e->n_maps * e->S, cfg->step_reward);
   } catch (const std::bad_alloc&) {
-    delete e;
     return fail(CRL_E_ALLOC, "host allocation failed");
   }
   auto bail = [&](hipError_t x, const char* what) {
-    delete e;
     return fail(CRL_E_DEVICE, "%s: %s", what, hipGetErrorString(x));
   };
   hipError_t h;
@@ -700,8 +708,91 @@ int crl_create(const crl_config* cfg, int device, crl_engine** out) {
                           hipMemcpyHostToDevice, e->stream)) != hipSuccess)
     return bail(h, "upload cell rewards");
   if ((h = hipStreamSynchronize(e->stream)) != hipSuccess) return bail(h, "sync");
-  *out = e;
+  *out = own.release();
   return CRL_OK;
+}
+
+int reset_envs(crl_engine* e, int32_t first, int32_t count) {
+  int rc = check_engine(e);
+  if (rc) return rc;
+  if (first < 0 || count < 0 || (int64_t)first + count > e->N)
+    return fail(CRL_E_RANGE, "env range [%d,%d) outside [0,%d)", first, first + count, e->N);
+  if (count == 0) return CRL_OK;
+  hipLaunchKernelGGL(crl::k_reset, dim3((count + 255) / 256), dim3(256), 0, e->stream, e->ptrs(), first,
+                     count);
+  HIP_TRY(hipGetLastError());
+  e->have_transition = false;
+  return CRL_OK;
+}
+
+int set_maps(crl_engine* e, const uint8_t* cell_class, const int32_t* start,
+                 const float* cell_reward) {
+  int rc = check_engine(e);
+  if (rc) return rc;
+  if (!cell_class) return fail(CRL_E_ARG, "cell_class is null");
+  const bool cells = (e->cfg.reward_flags & CRL_REWARD_CELLS) != 0;
+  if (cells && !cell_reward) return fail(CRL_E_ARG, "reward_flags asks for cell rewards but none given");
+  if (!cells && cell_reward) return fail(CRL_E_ARG, "cell rewards given but reward_flags has no CRL_REWARD_CELLS");
+  const size_t total = (size_t)e->n_maps * e->S;
+  for (size_t i = 0; i < total; ++i)
+    if (cell_class[i] > CRL_CELL_WALL) return fail(CRL_E_ARG, "cell_class[%zu] = %d is not a cell class", i, (int)cell_class[i]);
+  if (start)
+    for (int i = 0; i < e->N; ++i)
+      if (start[i] < 0 || (size_t)start[i] >= e->S)
+        return fail(CRL_E_RANGE, "start[%d] = %d outside [0,%zu)", i, start[i], e->S);
+  std::memcpy(e->h_class.data(), cell_class, total);
+  if (cells) std::memcpy(e->h_cell_reward.data(), cell_reward, total * sizeof(float));
+  rc = upload_maps(e);
+  if (rc) return rc;
+  if (start) {
+    HIP_TRY(hipMemcpyAsync(e->start.p, start, (size_t)e->N * 4, hipMemcpyHostToDevice, e->stream));
+    HIP_TRY(hipStreamSynchronize(e->stream));
+  }
+  return reset_envs(e, 0, e->N);
+}
+
+int set_cell(crl_engine* e, int32_t map_index, int32_t cell, int32_t cell_class,
+                 float cell_reward) {
+  int rc = check_engine(e);
+  if (rc) return rc;
+  if (map_index < 0 || map_index >= e->n_maps) return fail(CRL_E_RANGE, "map index %d outside [0,%d)", map_index, e->n_maps);
+  if (cell < 0 || (size_t)cell >= e->S) return fail(CRL_E_RANGE, "cell %d outside [0,%zu)", cell, e->S);
+  if (cell_class < CRL_CELL_FREE || cell_class > CRL_CELL_WALL) return fail(CRL_E_ARG, "%d is not a cell class", cell_class);
+  const size_t at = (size_t)map_index * e->S + cell;
+  e->h_class[at] = (uint8_t)cell_class;
+  const size_t word = (size_t)map_index * e->map_words + (cell >> 4);
+  uint32_t& packed = e->stage_word;  // outlives this call: the copy below is asynchronous
+  packed = 0;
+  const size_t first = (size_t)map_index * e->S + ((size_t)(cell >> 4) << 4);
+  for (size_t j = 0; j < 16 && ((size_t)(cell >> 4) << 4) + j < e->S; ++j)
+    packed |= (uint32_t)(e->h_class[first + j] & 3u) << (2 * j);
+  HIP_TRY(hipMemcpyAsync(e->map.p + word, &packed, 4, hipMemcpyHostToDevice, e->stream));
+  rc = build_moves(e, map_index, 1);  // the neighbours' codes name this cell
+  if (rc) return rc;
+  if (e->cfg.reward_flags & CRL_REWARD_CELLS) {
+    e->h_cell_reward[at] = cell_reward;
+    HIP_TRY(hipMemcpyAsync(e->cell_reward.p + at, &e->h_cell_reward[at], 4, hipMemcpyHostToDevice, e->stream));
+  }
+  HIP_TRY(hipStreamSynchronize(e->stream));
+  return CRL_OK;
+}
+
+}  // namespace
+
+extern "C" {
+
+const char* crl_last_error(void) { return g_err.c_str(); }
+const char* crl_version(void) { return CRL_VERSION; }
+
+int crl_device_count(void) {
+  int n = 0;
+  hipError_t e = hipGetDeviceCount(&n);
+  if (e != hipSuccess) return fail(CRL_E_DEVICE, "hipGetDeviceCount: %s", hipGetErrorString(e));
+  return n;
+}
+
+int crl_create(const crl_config* cfg, int device, crl_engine** out) {
+  return guarded([&] { return create_engine(cfg, device, out); });
 }
 
 int crl_destroy(crl_engine* e) {
@@ -756,67 +847,15 @@ int crl_sync(crl_engine* e) {
 
 int crl_set_maps(crl_engine* e, const uint8_t* cell_class, const int32_t* start,
                  const float* cell_reward) {
-  int rc = check_engine(e);
-  if (rc) return rc;
-  if (!cell_class) return fail(CRL_E_ARG, "cell_class is null");
-  const bool cells = (e->cfg.reward_flags & CRL_REWARD_CELLS) != 0;
-  if (cells && !cell_reward) return fail(CRL_E_ARG, "reward_flags asks for cell rewards but none given");
-  if (!cells && cell_reward) return fail(CRL_E_ARG, "cell rewards given but reward_flags has no CRL_REWARD_CELLS");
-  const size_t total = (size_t)e->n_maps * e->S;
-  for (size_t i = 0; i < total; ++i)
-    if (cell_class[i] > CRL_CELL_WALL) return fail(CRL_E_ARG, "cell_class[%zu] = %d is not a cell class", i, (int)cell_class[i]);
-  if (start)
-    for (int i = 0; i < e->N; ++i)
-      if (start[i] < 0 || (size_t)start[i] >= e->S)
-        return fail(CRL_E_RANGE, "start[%d] = %d outside [0,%zu)", i, start[i], e->S);
-  std::memcpy(e->h_class.data(), cell_class, total);
-  if (cells) std::memcpy(e->h_cell_reward.data(), cell_reward, total * sizeof(float));
-  rc = upload_maps(e);
-  if (rc) return rc;
-  if (start) {
-    HIP_TRY(hipMemcpyAsync(e->start.p, start, (size_t)e->N * 4, hipMemcpyHostToDevice, e->stream));
-    HIP_TRY(hipStreamSynchronize(e->stream));
-  }
-  return crl_reset(e, 0, e->N);
+  return guarded([&] { return set_maps(e, cell_class, start, cell_reward); });
 }
 
 int crl_set_cell(crl_engine* e, int32_t map_index, int32_t cell, int32_t cell_class,
                  float cell_reward) {
-  int rc = check_engine(e);
-  if (rc) return rc;
-  if (map_index < 0 || map_index >= e->n_maps) return fail(CRL_E_RANGE, "map index %d outside [0,%d)", map_index, e->n_maps);
-  if (cell < 0 || (size_t)cell >= e->S) return fail(CRL_E_RANGE, "cell %d outside [0,%zu)", cell, e->S);
-  if (cell_class < CRL_CELL_FREE || cell_class > CRL_CELL_WALL) return fail(CRL_E_ARG, "%d is not a cell class", cell_class);
-  const size_t at = (size_t)map_index * e->S + cell;
-  e->h_class[at] = (uint8_t)cell_class;
-  const size_t word = (size_t)map_index * e->map_words + (cell >> 4);
-  uint32_t packed = 0;
-  const size_t first = (size_t)map_index * e->S + ((size_t)(cell >> 4) << 4);
-  for (size_t j = 0; j < 16 && ((size_t)(cell >> 4) << 4) + j < e->S; ++j)
-    packed |= (uint32_t)(e->h_class[first + j] & 3u) << (2 * j);
-  HIP_TRY(hipMemcpyAsync(e->map.p + word, &packed, 4, hipMemcpyHostToDevice, e->stream));
-  rc = build_moves(e, map_index, 1);  // the neighbours' codes name this cell
-  if (rc) return rc;
-  if (e->cfg.reward_flags & CRL_REWARD_CELLS) {
-    e->h_cell_reward[at] = cell_reward;
-    HIP_TRY(hipMemcpyAsync(e->cell_reward.p + at, &cell_reward, 4, hipMemcpyHostToDevice, e->stream));
-  }
-  HIP_TRY(hipStreamSynchronize(e->stream));
-  return CRL_OK;
+  return guarded([&] { return set_cell(e, map_index, cell, cell_class, cell_reward); });
 }
 
-int crl_reset(crl_engine* e, int32_t first, int32_t count) {
-  int rc = check_engine(e);
-  if (rc) return rc;
-  if (first < 0 || count < 0 || (int64_t)first + count > e->N)
-    return fail(CRL_E_RANGE, "env range [%d,%d) outside [0,%d)", first, first + count, e->N);
-  if (count == 0) return CRL_OK;
-  hipLaunchKernelGGL(crl::k_reset, dim3((count + 255) / 256), dim3(256), 0, e->stream, e->ptrs(), first,
-                     count);
-  HIP_TRY(hipGetLastError());
-  e->have_transition = false;
-  return CRL_OK;
-}
+int crl_reset(crl_engine* e, int32_t first, int32_t count) { return reset_envs(e, first, count); }
 
 int crl_step(crl_engine* e, const int32_t* actions) {
   int rc = check_engine(e);
@@ -942,18 +981,26 @@ int crl_run_fused(crl_engine* e, int32_t n_steps) {
   if (n_steps == 0) return CRL_OK;
   if (e->cfg.table_mode == CRL_TABLE_PER_ENV) {
     const FusedPlan p = plan_fused(e, n_steps);
+    if (p.lds > kLdsPerWorkgroup)
+      return fail(CRL_E_STATE, "launch plan %s needs %zu bytes of LDS per workgroup, the device has %zu",
+                  p.name, p.lds, kLdsPerWorkgroup);
     if (p.tickets) {
       if (e->ticket.ensure(3) != hipSuccess) return fail(CRL_E_ALLOC, "ticket counter allocation failed");
       if (!e->hybrid_opt_in) {
+        // every instantiation launch_fused_a can pick: the plain ones, too, ask for
+        // more than the default 64 KB when large per-env maps share a workgroup
         const void* fns[] = {
-            reinterpret_cast<const void*>(&crl::k_fused_tickets<4, 1, true, false>),
-            reinterpret_cast<const void*>(&crl::k_fused_tickets<4, 0, true, false>),
-            reinterpret_cast<const void*>(&crl::k_fused_tickets<4, 1, false, true>),
-            reinterpret_cast<const void*>(&crl::k_fused_tickets<4, 2, false, true>),
-            reinterpret_cast<const void*>(&crl::k_fused_tickets<8, 1, true, false>),
-            reinterpret_cast<const void*>(&crl::k_fused_tickets<8, 0, true, false>),
-            reinterpret_cast<const void*>(&crl::k_fused_tickets<8, 1, false, true>),
-            reinterpret_cast<const void*>(&crl::k_fused_tickets<8, 2, false, true>)};
+#define CRL_TICKET_KERNELS(A)                                                          \
+  reinterpret_cast<const void*>(&crl::k_fused_tickets<A, 0, false, false>),            \
+      reinterpret_cast<const void*>(&crl::k_fused_tickets<A, 1, false, false>),        \
+      reinterpret_cast<const void*>(&crl::k_fused_tickets<A, 2, false, false>),        \
+      reinterpret_cast<const void*>(&crl::k_fused_tickets<A, 0, true, false>),         \
+      reinterpret_cast<const void*>(&crl::k_fused_tickets<A, 1, true, false>),         \
+      reinterpret_cast<const void*>(&crl::k_fused_tickets<A, 1, false, true>),         \
+      reinterpret_cast<const void*>(&crl::k_fused_tickets<A, 2, false, true>)
+            CRL_TICKET_KERNELS(4), CRL_TICKET_KERNELS(8)
+#undef CRL_TICKET_KERNELS
+        };
         for (const void* fn : fns)
           HIP_TRY(hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, (int)kLdsPerWorkgroup));
         e->hybrid_opt_in = true;
@@ -1140,11 +1187,11 @@ int crl_device_ptr(crl_engine* e, int32_t which, void** out) {
   return CRL_OK;
 }
 
-int crl_fused_kernel_info(crl_engine* e, char* name, size_t name_len, int32_t* grid, int32_t* block,
-                          int32_t* lds_bytes) {
+int crl_fused_kernel_info(crl_engine* e, int32_t n_steps, char* name, size_t name_len, int32_t* grid,
+                          int32_t* block, int32_t* lds_bytes) {
   if (!e) return fail(CRL_E_ARG, "null engine");
   if (e->cfg.table_mode == CRL_TABLE_PER_ENV) {
-    const FusedPlan p = plan_fused(e, 1 << 20);  // the plan of a long launch
+    const FusedPlan p = plan_fused(e, n_steps > 0 ? n_steps : 1 << 20);  // <= 0: a long launch
     if (name && name_len) snprintf(name, name_len, "%s", p.name);
     if (grid) *grid = p.grid;
     if (block) *block = p.block;
@@ -1155,6 +1202,23 @@ int crl_fused_kernel_info(crl_engine* e, char* name, size_t name_len, int32_t* g
     if (block) *block = 256;
     if (lds_bytes) *lds_bytes = e->map_words * 4;
   }
+  return CRL_OK;
+}
+
+int crl_fused_plan_for_config(const crl_config* cfg, int32_t n_steps, char* name, size_t name_len,
+                              int32_t* grid, int32_t* block, int32_t* lds_bytes) {
+  int rc = crl::validate_config(cfg, g_err);
+  if (rc != CRL_OK) return rc;
+  if (cfg->table_mode != CRL_TABLE_PER_ENV) return fail(CRL_E_ARG, "only per-env tables have a fused launch plan");
+  crl_engine shell;  // sizes only: nothing is allocated and no device is touched
+  set_geometry(&shell, *cfg);
+  const FusedPlan p = plan_fused(&shell, n_steps > 0 ? n_steps : 1 << 20);
+  if (name && name_len) snprintf(name, name_len, "%s", p.name);
+  if (grid) *grid = p.grid;
+  if (block) *block = p.block;
+  if (lds_bytes) *lds_bytes = (int32_t)p.lds;
+  if (p.grid < 1 || p.block < 64 || p.block > 1024 || p.lds > kLdsPerWorkgroup)
+    return fail(CRL_E_STATE, "launch plan %s: grid %d, block %d, %zu bytes of LDS", p.name, p.grid, p.block, p.lds);
   return CRL_OK;
 }
 
@@ -1171,6 +1235,14 @@ int crl_probe_copy(size_t n_bytes, int repeats) {
                        reinterpret_cast<const uint4*>(src.p), reinterpret_cast<uint4*>(dst.p), n16);
   HIP_TRY(hipGetLastError());
   HIP_TRY(hipDeviceSynchronize());
+  // the copy arrived: both ends of the destination hold the source's pattern
+  uint8_t ends[2][256];
+  const size_t tail = n_bytes >= sizeof ends[0] ? n_bytes - sizeof ends[0] : 0;
+  const size_t len = n_bytes >= sizeof ends[0] ? sizeof ends[0] : n_bytes;
+  HIP_TRY(hipMemcpy(ends[0], dst.p, len, hipMemcpyDeviceToHost));
+  HIP_TRY(hipMemcpy(ends[1], dst.p + tail, len, hipMemcpyDeviceToHost));
+  for (size_t i = 0; i < len; ++i)
+    if (ends[0][i] != 1 || ends[1][i] != 1) return fail(CRL_E_DEVICE, "copy kernel left byte %zu unwritten", i);
   return CRL_OK;
 }
 

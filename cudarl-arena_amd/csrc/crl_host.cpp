@@ -3,6 +3,7 @@
 #include "crl_host.h"
 
 #include <algorithm>
+#include <atomic>
 #include <cmath>
 #include <cstdio>
 #include <cstring>
@@ -101,22 +102,35 @@ struct WordStream {
   }
 };
 
+// f(i) for i in [0, n) on up to 16 threads.  Nothing escapes: false if f, or
+// starting a thread, threw (the C ABI above never lets an exception through).
 template <class F>
-void parallel_for(int n, F f) {
+bool parallel_for(int n, F f) {
   unsigned hw = std::thread::hardware_concurrency();
   int workers = (int)std::min<unsigned>(hw ? hw : 1u, 16u);
   if (n < 4096) workers = 1;
+  std::atomic<bool> ok{true};
+  auto run = [&](int lo, int hi) {
+    try {
+      for (int i = lo; i < hi; ++i) f(i);
+    } catch (...) {
+      ok = false;
+    }
+  };
   if (workers <= 1) {
-    for (int i = 0; i < n; ++i) f(i);
-    return;
+    run(0, n);
+    return ok;
   }
   std::vector<std::thread> pool;
-  for (int w = 0; w < workers; ++w)
-    pool.emplace_back([=] {
-      const int lo = (int)((int64_t)n * w / workers), hi = (int)((int64_t)n * (w + 1) / workers);
-      for (int i = lo; i < hi; ++i) f(i);
-    });
+  try {
+    pool.reserve((size_t)workers);
+    for (int w = 0; w < workers; ++w)
+      pool.emplace_back(run, (int)((int64_t)n * w / workers), (int)((int64_t)n * (w + 1) / workers));
+  } catch (...) {
+    ok = false;  // the threads already started still finish their share
+  }
   for (auto& t : pool) t.join();
+  return ok;
 }
 
 // index of the j-th FREE cell
@@ -151,10 +165,14 @@ void crl_explore_draw(uint64_t seed, uint32_t env, uint64_t t, int32_t n_actions
 int crl_eps_table(const crl_config* cfg, float* out, int32_t cap, int32_t* len) {
   std::string why;
   if (crl::validate_config(cfg, why) != CRL_OK) return CRL_E_ARG;
-  const std::vector<float> tab = crl::build_eps_table(*cfg);
-  if (len) *len = (int32_t)tab.size();
-  if (out)
-    for (int32_t i = 0; i < cap && (size_t)i < tab.size(); ++i) out[i] = tab[(size_t)i];
+  try {
+    const std::vector<float> tab = crl::build_eps_table(*cfg);
+    if (len) *len = (int32_t)tab.size();
+    if (out)
+      for (int32_t i = 0; i < cap && (size_t)i < tab.size(); ++i) out[i] = tab[(size_t)i];
+  } catch (...) {
+    return CRL_E_ALLOC;
+  }
   return CRL_OK;
 }
 
@@ -189,8 +207,9 @@ int crl_gen_maps_bernoulli(uint64_t seed, int32_t n_maps, int32_t n_envs, int32_
   if (n_maps != 1 && n_maps != n_envs) return CRL_E_ARG;
   const int S = width * height;
   if (S < 2) return CRL_E_ARG;
+  try {
   std::vector<int> n_free((size_t)n_maps), goal((size_t)n_maps);
-  crl::parallel_for(n_maps, [&](int m) {
+  bool ok = crl::parallel_for(n_maps, [&](int m) {
     uint8_t* cls = cell_class + (size_t)m * S;
     crl::WordStream walls(seed, (uint32_t)m, crl::kStreamMap);
     crl::WordStream traps(seed, (uint32_t)m, crl::kStreamTrap);
@@ -224,12 +243,15 @@ int crl_gen_maps_bernoulli(uint64_t seed, int32_t n_maps, int32_t n_envs, int32_
     for (int c = 0; c < S; ++c)
       if (cls[c] == CRL_CELL_FREE) free_cells.push_back(c);
     const uint32_t nf = (uint32_t)free_cells.size();
-    crl::parallel_for(n_envs, [&](int i) {
+    ok = crl::parallel_for(n_envs, [&](int i) {
       crl::WordStream sg(seed, (uint32_t)i, crl::kStreamStartGoal);
       start[i] = free_cells[crl::below(sg.word(4), nf)];
-    });
+    }) && ok;
   }
-  return CRL_OK;
+  return ok ? CRL_OK : CRL_E_ALLOC;
+  } catch (...) {
+    return CRL_E_ALLOC;
+  }
 }
 
 int crl_gen_maps_noise(uint64_t seed, int32_t n_maps, int32_t width, int32_t height, int32_t pitch,
@@ -240,7 +262,7 @@ int crl_gen_maps_noise(uint64_t seed, int32_t n_maps, int32_t width, int32_t hei
   const int S = width * height;
   if (S < 2) return CRL_E_ARG;
   const int lw = (width + pitch - 1) / pitch + 1, lh = (height + pitch - 1) / pitch + 1;
-  crl::parallel_for(n_maps, [&](int m) {
+  const bool ok = crl::parallel_for(n_maps, [&](int m) {
     uint8_t* cls = cell_class + (size_t)m * S;
     crl::WordStream lat(seed, (uint32_t)m, crl::kStreamLattice);
     std::vector<float> lattice((size_t)lw * lh);
@@ -287,7 +309,7 @@ int crl_gen_maps_noise(uint64_t seed, int32_t n_maps, int32_t width, int32_t hei
       cr[g] += goal_bonus;
     }
   });
-  return CRL_OK;
+  return ok ? CRL_OK : CRL_E_ALLOC;
 }
 
 }  // extern "C"

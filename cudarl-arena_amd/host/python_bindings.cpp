@@ -10,6 +10,7 @@
 #include <stdexcept>
 
 #include "batched_environment.h"
+#include "environment.h"
 #include "environment_bridge.h"
 #include "npy.h"
 #include "q_learning.h"
@@ -103,10 +104,54 @@ py::array_t<T> to_array(const std::vector<T>& v) {
   return a;
 }
 
+// The reference's other Python surface (src/bindings/python_bindings.cpp:9-63,
+// class PyEnvironment bound as `Environment` there): observations as an (H, W)
+// numpy array, a dict for info, width / height / env_id as read-only properties.
+// Bound here under its C++ name beside the current `Environment`.
+class PyEnvironment {
+ public:
+  PyEnvironment(int width, int height, int env_id = 0)
+      : width_(width), height_(height), env_id_(env_id), env_(env_id, width, height) {}
+
+  py::array_t<float> reset() {
+    env_.reset();
+    return observation();
+  }
+  std::tuple<py::array_t<float>, float, bool, py::dict> step(int action) {
+    env_.step(action);
+    py::dict info;
+    info["agent_x"] = env_.getAgentX();
+    info["agent_y"] = env_.getAgentY();
+    return std::make_tuple(observation(), env_.getReward(), env_.isDone(), info);
+  }
+  py::array_t<float> observation() const {
+    const std::vector<float> grid = env_.getGrid();  // row-major [y][x]: already the (H, W) layout
+    py::array_t<float> obs({(py::ssize_t)height_, (py::ssize_t)width_});
+    std::memcpy(obs.mutable_data(), grid.data(), grid.size() * sizeof(float));
+    return obs;
+  }
+  int width() const { return width_; }
+  int height() const { return height_; }
+  int env_id() const { return env_id_; }
+
+ private:
+  int width_, height_, env_id_;
+  Environment env_;
+};
+
 }  // namespace
 
 PYBIND11_MODULE(cudarl_core, m) {
   m.doc() = "CudaRL-Arena Python bindings (MI355X engine)";
+
+  py::class_<PyEnvironment>(m, "PyEnvironment")
+      .def(py::init<int, int, int>(), py::arg("width") = 10, py::arg("height") = 10, py::arg("env_id") = 0)
+      .def("reset", &PyEnvironment::reset)
+      .def("step", &PyEnvironment::step)
+      .def("get_observation", &PyEnvironment::observation)
+      .def_property_readonly("width", &PyEnvironment::width)
+      .def_property_readonly("height", &PyEnvironment::height)
+      .def_property_readonly("env_id", &PyEnvironment::env_id);
 
   py::class_<EnvironmentBridge>(m, "Environment")
       .def(py::init<int, int>(), py::arg("width") = 10, py::arg("height") = 10)
@@ -123,7 +168,7 @@ PYBIND11_MODULE(cudarl_core, m) {
   py::class_<CudaQLearning>(m, "CudaQLearning")
       .def(py::init<int, int, int, float, float, int>(), py::arg("width"), py::arg("height"),
            py::arg("action_space_size"), py::arg("learning_rate") = 0.1f,
-           py::arg("discount_factor") = 0.99f, py::arg("max_mode") = 0)
+           py::arg("discount_factor") = 0.99f, py::arg("max_mode") = 1)
       .def("update_batch", &CudaQLearning::update_batch)
       .def("get_q_table", &CudaQLearning::get_q_table)
       .def("set_q_table", &CudaQLearning::set_q_table)

@@ -8,10 +8,13 @@ struct crl_engine;
 
 class CudaQLearning {
  public:
-  // max_mode (additive, default 0): 0 = true max over the next row
-  // (src/gpu/kernels.cu:35-45), 1 = max seeded with 0 (src/kernels.cu:101-110)
+  // max_mode (additive): 1 = max over the next row seeded with 0, which is what the
+  // kernel behind this class upstream computes (update_q_values_kernel,
+  // src/kernels.cu:101-110) and therefore the default of the five-argument
+  // constructor; 0 = the true max (src/gpu/kernels.cu:35-45, np.max in src/train.py:134),
+  // the default of the batched engine and of train().
   CudaQLearning(int width, int height, int action_space_size, float learning_rate = 0.1f,
-                float discount_factor = 0.99f, int max_mode = 0);
+                float discount_factor = 0.99f, int max_mode = 1);
   ~CudaQLearning();
   CudaQLearning(const CudaQLearning&) = delete;
   CudaQLearning& operator=(const CudaQLearning&) = delete;

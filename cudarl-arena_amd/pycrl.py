@@ -86,7 +86,7 @@ EXPORTS = [
     "crl_step", "crl_select", "crl_update", "crl_td_update", "crl_run_fused", "crl_get_state",
     "crl_set_state", "crl_get_episode_stats", "crl_get_step_count", "crl_set_step_count", "crl_q_get", "crl_q_set",
     "crl_q_get_range", "crl_set_trace", "crl_get_trace", "crl_set_exploration_stream",
-    "crl_device_ptr", "crl_fused_kernel_info", "crl_philox4x32_10", "crl_explore_draw",
+    "crl_device_ptr", "crl_fused_kernel_info", "crl_fused_plan_for_config", "crl_philox4x32_10", "crl_explore_draw",
     "crl_eps_table", "crl_gen_maps_bernoulli", "crl_gen_maps_noise", "crl_probe_copy",
 ]
 
@@ -131,8 +131,10 @@ def load():
     lib.crl_get_trace.argtypes = [vp, i32, vp, vp, vp, vp]
     lib.crl_set_exploration_stream.argtypes = [vp, i32, vp, vp]
     lib.crl_device_ptr.argtypes = [vp, i32, C.POINTER(vp)]
-    lib.crl_fused_kernel_info.argtypes = [vp, C.c_char_p, C.c_size_t, C.POINTER(i32), C.POINTER(i32),
+    lib.crl_fused_kernel_info.argtypes = [vp, i32, C.c_char_p, C.c_size_t, C.POINTER(i32), C.POINTER(i32),
                                           C.POINTER(i32)]
+    lib.crl_fused_plan_for_config.argtypes = [C.POINTER(Config), i32, C.c_char_p, C.c_size_t, C.POINTER(i32),
+                                              C.POINTER(i32), C.POINTER(i32)]
     lib.crl_philox4x32_10.argtypes = [vp, vp, vp]
     lib.crl_philox4x32_10.restype = None
     lib.crl_explore_draw.argtypes = [u64, C.c_uint32, u64, i32, C.POINTER(f32), C.POINTER(i32)]
@@ -181,6 +183,14 @@ def eps_table(cfg):
     out = np.empty(n.value, np.float32)
     _check(load().crl_eps_table(C.byref(cfg), _ptr(out), n.value, C.byref(n)))
     return out
+
+
+def fused_plan_for_config(cfg, n_steps=0):
+    """Launch plan of crl_run_fused(n_steps) for an engine made from cfg (host only)."""
+    name = C.create_string_buffer(128)
+    g, b, l = C.c_int32(), C.c_int32(), C.c_int32()
+    _check(load().crl_fused_plan_for_config(C.byref(cfg), n_steps, name, 128, C.byref(g), C.byref(b), C.byref(l)))
+    return dict(name=name.value.decode(), grid=g.value, block=b.value, lds_bytes=l.value)
 
 
 def classify_grid(grid, step_reward=-0.01):
@@ -348,8 +358,9 @@ class Engine:
         _check(self.lib.crl_device_ptr(self.h, which, C.byref(p)))
         return p.value
 
-    def fused_kernel_info(self):
+    def fused_kernel_info(self, n_steps=0):
+        """Plan of crl_run_fused(n_steps); 0 = a long launch."""
         name = C.create_string_buffer(128)
         g, b, l = C.c_int32(), C.c_int32(), C.c_int32()
-        _check(self.lib.crl_fused_kernel_info(self.h, name, 128, C.byref(g), C.byref(b), C.byref(l)))
+        _check(self.lib.crl_fused_kernel_info(self.h, n_steps, name, 128, C.byref(g), C.byref(b), C.byref(l)))
         return dict(name=name.value.decode(), grid=g.value, block=b.value, lds_bytes=l.value)

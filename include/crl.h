@@ -9,6 +9,11 @@
  * the caller; there is no CPU fallback: without a usable HIP device
  * `crl_create` fails with CRL_E_DEVICE.
  *
+ * Built for MI355X only: the launch plans assume its 256 compute units, 160 KB
+ * of LDS per workgroup and 256 MB last-level cache as compile-time constants
+ * (they are not read from hipDeviceProp_t); on another gfx950 part results stay
+ * the same and only the tuning is off.
+ *
  * Citations name the file:line of life423/CudaRL-Arena that the entry point
  * replaces.  State index is s = y*W + x and the table layout is
  * Q[s*A + a], fp32 (src/kernels.cu:96, src/q_learning.cu:196).
@@ -237,10 +242,18 @@ enum {
 };
 int crl_device_ptr(crl_engine* e, int32_t which, void** out);
 
-/* name and launch geometry of the kernel crl_run_fused uses for this engine on a
- * long launch (launches of fewer than 64 steps keep every table in HBM) */
-int crl_fused_kernel_info(crl_engine* e, char* name, size_t name_len, int32_t* grid,
-                          int32_t* block, int32_t* lds_bytes);
+/* name and launch geometry of the kernel crl_run_fused(e, n_steps) would use for
+ * this engine (the plan depends on the launch length: short launches keep every
+ * table in HBM and every env in flight).  n_steps <= 0 asks for the plan of a
+ * long launch. */
+int crl_fused_kernel_info(crl_engine* e, int32_t n_steps, char* name, size_t name_len,
+                          int32_t* grid, int32_t* block, int32_t* lds_bytes);
+
+/* The same for an engine that crl_create(cfg) would make, without making one
+ * (host only, needs no device): CRL_E_STATE if the plan does not fit the device's
+ * limits (160 KB of LDS per workgroup).  Per-env tables only. */
+int crl_fused_plan_for_config(const crl_config* cfg, int32_t n_steps, char* name, size_t name_len,
+                              int32_t* grid, int32_t* block, int32_t* lds_bytes);
 
 /* Measurement helper (no reference counterpart): one launch of a plain copy
  * kernel `k_probe_copy` moving n_bytes from one device buffer to another, so

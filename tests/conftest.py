@@ -178,9 +178,9 @@ class Oracle:
         return tr
 
 
-def oracle_run_slice(orc, cfg, lo, hi, cls, start, t0, n_steps):
+def oracle_run_slice(orc, cfg, lo, hi, cls, start, t0, n_steps, cr=None):
     """Oracle results for envs [lo, hi) of a larger per-env-table batch (envs are
-    independent and the draws are keyed by the global env index).  cls / start
+    independent and the draws are keyed by the global env index).  cls / start / cr
     hold only the slice.  Returns (Q[hi-lo, S, A], state dict of the slice)."""
     n = hi - lo
     S, A = cfg.width * cfg.height, cfg.n_actions
@@ -190,12 +190,14 @@ def oracle_run_slice(orc, cfg, lo, hi, cls, start, t0, n_steps):
               reward=np.zeros(n, np.float32), done=np.zeros(n, np.uint8), action=np.zeros(n, np.uint8))
     cls = np.ascontiguousarray(cls, np.uint8)
     start = np.ascontiguousarray(start, np.int32)
+    cr = None if cr is None else np.ascontiguousarray(cr, np.float32)
 
     def shifted(a, per_env_bytes):  # address such that index `lo` lands on a[0]
         return C.c_void_p(a.ctypes.data - lo * per_env_bytes)
 
     per_map = 0 if cfg.map_mode == 1 else S
-    rc = orc.lib.orc_run_range(C.byref(cfg), lo, hi, shifted(cls, per_map), None, shifted(start, 4),
+    rc = orc.lib.orc_run_range(C.byref(cfg), lo, hi, shifted(cls, per_map),
+                               None if cr is None else shifted(cr, per_map * 4), shifted(start, 4),
                                shifted(Q, K * 4), shifted(st["s"], 4), shifted(st["ep_step"], 4),
                                shifted(st["episode"], 4), shifted(st["reward"], 4), shifted(st["done"], 1),
                                shifted(st["action"], 1), t0, n_steps)

@@ -117,6 +117,91 @@ def test_noise_maps(pycrl):
     assert same_right > 0.9
 
 
+def test_noise_map_matches_a_hand_worked_restatement(pycrl, oracle):
+    """One tiny value-noise map recomputed from the Philox words up: lattice values,
+    smoothstep-bilinear cell values, the k highest as walls, goal and start among
+    the free cells, Box-Muller rewards of two known words.  A wrong lattice index,
+    a swapped interpolation axis or a sign slip in the rewards changes it."""
+    seed, W, H, pitch, frac, sigma, bonus = 11, 6, 5, 4, 0.3, 0.05, 10.0
+    cls, start, cr = pycrl.gen_maps_noise(seed, 2, W, H, pitch, frac, sigma, bonus)
+    f32 = np.float32
+    for m in range(2):
+        def word(stream, i):  # counter (map, stream id, i // 4, 0), key = seed
+            return int(oracle.philox([m, stream, i // 4, 0], [seed & 0xFFFFFFFF, seed >> 32])[i % 4])
+        lw, lh = (W + pitch - 1) // pitch + 1, (H + pitch - 1) // pitch + 1
+        assert (lw, lh) == (3, 3)
+        lat = np.array([f32(word(5, i) >> 8) * f32(2.0 ** -24) for i in range(lw * lh)], f32).reshape(lh, lw)
+        val = np.zeros((H, W), f32)
+        for y in range(H):
+            for x in range(W):
+                gx, gy = x // pitch, y // pitch
+                fx, fy = f32(x % pitch) / f32(pitch), f32(y % pitch) / f32(pitch)
+                fx = fx * fx * (f32(3) - f32(2) * fx)
+                fy = fy * fy * (f32(3) - f32(2) * fy)
+                top = lat[gy, gx] + (lat[gy, gx + 1] - lat[gy, gx]) * fx
+                bot = lat[gy + 1, gx] + (lat[gy + 1, gx + 1] - lat[gy + 1, gx]) * fx
+                val[y, x] = top + (bot - top) * fy
+        # corners of a lattice square reproduce the lattice values exactly
+        assert val[0, 0] == lat[0, 0] and val[4, 4] == lat[1, 1] and val[0, 4] == lat[0, 1]
+        n_wall = int(frac * W * H)
+        assert n_wall == 9
+        order = sorted(range(W * H), key=lambda c: (-val.ravel()[c], c))
+        want = np.zeros(W * H, np.uint8)
+        want[order[:n_wall]] = 3
+        free = [c for c in range(W * H) if want[c] == 0]
+        goal = free[(word(2, 0) * len(free)) >> 32]
+        want[goal] = 1
+        free.remove(goal)
+        assert start[m] == free[(word(2, 1) * len(free)) >> 32]
+        assert np.array_equal(cls[m], want)
+        for c in range(0, W * H, 2):
+            u1 = (f32(word(4, c) >> 8) + f32(1)) * f32(2.0 ** -24)
+            u2 = f32(word(4, c + 1) >> 8) * f32(2.0 ** -24)
+            rad = np.sqrt(f32(-2) * np.log(u1, dtype=f32), dtype=f32)
+            ang = f32(6.28318530717958647692) * u2
+            pair = [sigma * rad * np.cos(ang, dtype=f32), sigma * rad * np.sin(ang, dtype=f32)]
+            for j in (0, 1):
+                if c + j < W * H:
+                    got = cr[m, c + j] - (bonus if c + j == goal else 0.0)
+                    assert abs(got - pair[j]) <= 2e-6, (m, c + j)
+        assert cr[m, goal] > 9.0
+
+
+def test_every_valid_configuration_has_a_launch_plan_that_fits(pycrl):
+    """The fused launch plan over a grid of shapes, host only: at most 160 KB of
+    LDS per workgroup and a non-empty grid, also where large per-env maps leave
+    room for fewer waves per workgroup than the planner would like."""
+    checked = 0
+    for A in (4, 8):
+        for W, H in ((4, 4), (16, 16), (32, 32), (33, 33), (40, 40), (48, 48), (64, 64), (65, 65), (128, 96),
+                     (256, 256)):
+            for N in (1, 100, 4096, 16384, 65536, 131072, 262144, 1 << 20):
+                if N * W * H * A * 4 > 64 << 30:
+                    continue
+                for n_steps in (1, 8, 20, 64, 128, 1000):
+                    for kw in (dict(), dict(eps_mode=pycrl.EPS_EPISODE_LINEAR, eps0=1.0, eps_end=0.1, eps_span=10),
+                               dict(goal_mode=pycrl.GOAL_ON_RESULT)):
+                        cfg = pycrl.make_config(N, W, H, n_actions=A, episode_len=128, **kw)
+                        plan = pycrl.fused_plan_for_config(cfg, n_steps)  # raises on a plan that does not fit
+                        assert 0 <= plan["lds_bytes"] <= 160 * 1024, (N, W, H, A, n_steps, plan)
+                        assert plan["grid"] >= 1 and plan["block"] in (64, 128, 192, 256, 320), plan
+                        checked += 1
+    assert checked > 2000
+    # the two cases that used to ask for 192 KB and 256 KB
+    for N, n in ((131072, 1000), (65536, 8)):
+        plan = pycrl.fused_plan_for_config(pycrl.make_config(N, 64, 64, episode_len=128), n)
+        assert plan["lds_bytes"] == 128 * 1024 and plan["block"] == 128
+    # the tuned configurations keep their plans
+    c4 = pycrl.make_config(1 << 20, 16, 16, episode_len=128, gamma=0.95)
+    assert pycrl.fused_plan_for_config(c4, 1000) == dict(name="k_fused_tickets<4,fast,hbm+lds>", grid=256, block=256,
+                                                         lds_bytes=152064)
+    c2 = pycrl.make_config(4096, 32, 32, episode_len=256)
+    assert pycrl.fused_plan_for_config(c2, 10000) == dict(name="k_fused_tickets<4,fast,hbm>", grid=128, block=64,
+                                                          lds_bytes=65536)
+    with pytest.raises(pycrl.CrlError):
+        pycrl.fused_plan_for_config(pycrl.make_config(64, 8, 8, table_mode=pycrl.TABLE_SHARED), 10)
+
+
 def test_npy_agent_files_match_numpy(pycrl, tmp_path):
     """QTableAgent.save / load files (src/train.py:150-168): float64 (W, H, A)
     indexed [x, y, a], exchanged with numpy in both directions."""

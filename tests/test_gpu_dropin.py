@@ -190,6 +190,24 @@ def test_q_learning_update_batch_matches_oracle(core, oracle, mode):
     assert q.get_best_action(2, 3) == best
 
 
+def test_q_learning_default_is_the_zero_floored_max_of_the_built_kernel(core):
+    """The five-argument constructor behaves like the class it replaces: the kernel
+    the reference builds seeds the max with 0.0f (src/kernels.cu:101-110), so an
+    all-negative next row bootstraps from 0, not from its largest entry; the true
+    max (src/gpu/kernels.cu:35-45) is the sixth argument's 0."""
+    r = -0.01
+    table = np.zeros((9, 4), np.float32)
+    table[4] = [-0.5, -0.25, -0.75, -1.0]  # next state (1,1): all negative, max -0.25
+    for args, m in (((3, 3, 4, 0.1, 0.99), np.float32(0.0)), ((3, 3, 4, 0.1, 0.99, 1), np.float32(0.0)),
+                    ((3, 3, 4, 0.1, 0.99, 0), np.float32(-0.25))):
+        q = core.CudaQLearning(*args)
+        q.set_q_table(table.ravel().tolist())
+        q.update_batch([(0, 0)], [2], [r], [(1, 1)], [False])
+        want = 0.1 * (-0.01 + 0.99 * float(m))  # from Q = 0: -0.001 floored, -0.02575 with the true max
+        got = q.get_q_value(0, 0, 2)
+        assert abs(got - want) <= 1e-8, (args, got, want)
+
+
 def test_q_learning_errors(core):  # src/q_learning.cu:117-124,181-183,192-194,212-214
     q = core.CudaQLearning(4, 4, 4)
     with pytest.raises(RuntimeError, match="Batch size exceeds maximum batch size"):
@@ -372,3 +390,70 @@ def test_train_cli_many_envs(gpu):
     assert "Evaluation episode 1: Reward = 0.94, Length = 7" in lines  # (4,4) -> (7,0)
     done = [l for l in lines if l.startswith("Done!")][0]
     assert int(done.split("(")[1].split()[0]) > 3000 * 50 * 7
+
+
+# ---- the demo and the device check (the reference's cudarl_app / cuda_test targets) ----
+
+def test_cudarl_app_demo_follows_the_step_rule(gpu):
+    """src/main.cu:21-99: ten random steps from the centre of the default 10x10
+    world, one update_batch, then Q(0,0,.) - which stays 0 because (0,0) cannot be
+    reached in ten steps (src/main.cu:92-94)."""
+    import re
+    import subprocess
+    out = subprocess.run([os.path.join(LIBDIR, "cudarl_app")], capture_output=True, text=True, timeout=100)
+    assert out.returncode == 0, out.stderr
+    lines = out.stdout.splitlines()
+    steps = [re.match(r"Step (\d+): Agent at \((\d+),(\d+)\), action (\d)", l) for l in lines]
+    steps = [m for m in steps if m]
+    after = [re.match(r"  New position: \((\d+),(\d+)\), Reward: (\S+), Done: (true|false)", l) for l in lines]
+    after = [m for m in after if m]
+    assert 1 <= len(steps) <= 10 and len(after) == len(steps)
+    x, y = 5, 5  # src/environment.cu:9-10
+    for k, (m, n) in enumerate(zip(steps, after)):
+        assert (int(m.group(1)), int(m.group(2)), int(m.group(3))) == (k, x, y)
+        dx, dy = {0: (0, -1), 1: (1, 0), 2: (0, 1), 3: (-1, 0)}[int(m.group(4))]  # src/kernels.cu:15-23
+        if 0 <= x + dx < 10 and 0 <= y + dy < 10:
+            x, y = x + dx, y + dy
+        assert (int(n.group(1)), int(n.group(2))) == (x, y)
+        goal = (x, y) == (9, 0)
+        assert float(n.group(3)) == (1.0 if goal else -0.01) and n.group(4) == ("true" if goal else "false")
+    assert [l for l in lines if l.startswith("  Q(0,0,")] == ["  Q(0,0,%d) = 0" % a for a in range(4)]
+
+
+def test_hip_test_sees_a_device_and_copies(gpu):
+    """The counterpart of the reference's cuda_test (src/cuda_test.cu:95-186: device
+    properties and a checked vector add): device count and a checked copy kernel."""
+    import re
+    import subprocess
+    out = subprocess.run([os.path.join(LIBDIR, "hip_test")], capture_output=True, text=True, timeout=100)
+    assert out.returncode == 0, out.stdout + out.stderr
+    m = re.match(r"(\d+) HIP device\(s\); engine version 0\.1\.0", out.stdout)
+    assert m and int(m.group(1)) >= 1
+    assert "copy kernel ok" in out.stdout
+
+
+# ---- the numpy-observation binding of src/bindings/python_bindings.cpp:9-80 -----------
+
+def test_numpy_observation_binding(core):
+    """tests/test_environment.py:17-66 restated on the bound class: (5,5) float
+    observation, return types of step, info with the agent's position; plus what
+    the stubbed upstream wrapper could not check - the dynamics."""
+    env = core.PyEnvironment(width=5, height=5)
+    assert (env.width, env.height, env.env_id) == (5, 5, 0)
+    with pytest.raises(AttributeError):
+        env.width = 3
+    obs = env.reset()
+    assert isinstance(obs, np.ndarray) and obs.shape == (5, 5) and obs.dtype == np.float32
+    assert obs[0, 4] == 1.0 and (np.delete(obs.ravel(), 4) <= 0.5).all()  # src/environment.cu:143-146
+    obs2, reward, done, info = env.step(1)  # right, from the centre (2,2)
+    assert isinstance(obs2, np.ndarray) and isinstance(reward, float) and isinstance(done, bool)
+    assert isinstance(info, dict) and obs2.shape == (5, 5) and np.array_equal(obs2, obs)
+    assert reward < 0 and abs(reward + 0.01) < 1e-7 and done is False
+    assert info == {"agent_x": 3, "agent_y": 2}
+    for a in (1, 0, 0):  # tests/test_environment.cpp:107-119: R,R,U,U reaches (4,0)
+        obs2, reward, done, info = env.step(a)
+    assert done is True and reward == 1.0 and info == {"agent_x": 4, "agent_y": 0}
+    assert np.array_equal(env.get_observation(), obs)
+    wide = core.PyEnvironment(7, 3, 9)
+    assert (wide.width, wide.height, wide.env_id) == (7, 3, 9) and wide.reset().shape == (3, 7)
+    assert core.PyEnvironment().reset().shape == (10, 10)

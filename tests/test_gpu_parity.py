@@ -400,6 +400,44 @@ def test_shared_table_run_to_run_identity(gpu):
     assert np.count_nonzero(qs[0]) > 100
 
 
+# ---- checkpoint / resume -------------------------------------------------------------
+
+@pytest.mark.parametrize("shared", [False, True])
+def test_resume_from_saved_state_equals_uninterrupted_run(gpu, shared):
+    """(tables, s, ep_step, episode, step count) is a complete resume state (the
+    exploration stream is counter-based): a fresh engine loaded with what a first
+    one held mid-run (src/q_learning.cu:176-189 get/set_q_table; src/train.py:150-168
+    save/load) ends bit-identical to a run that was never interrupted."""
+    N, W, H, first, rest = 1500, 12, 12, 333, 412  # an odd split: the Philox block of a step pair is cut
+    cls, start = gpu.gen_maps_bernoulli(9, 1 if shared else N, N, W, H, 0.15, 0.0 if shared else 0.03)
+    kw = dict(table_mode=gpu.TABLE_SHARED, map_mode=gpu.MAP_SHARED, lr=0.002, eps0=0.2) if shared else \
+        dict(eps_mode=gpu.EPS_EPISODE_LINEAR, eps0=0.9, eps_end=0.05, eps_span=6, lr=0.1)
+    cfg = gpu.make_config(N, W, H, episode_len=40, seed=17, **kw)
+    n_tables = 1 if shared else N
+    with gpu.Engine(cfg, 0) as eng:
+        eng.set_maps(cls, start)
+        eng.run_fused(first + rest)
+        want_st, want_q = eng.get_state(), eng.q_get(0, n_tables)
+    with gpu.Engine(cfg, 0) as eng:
+        eng.set_maps(cls, start)
+        eng.run_fused(first)
+        saved_st, saved_q, saved_t = eng.get_state(), eng.q_get(0, n_tables).copy(), eng.step_count
+    assert saved_t == first
+    with gpu.Engine(cfg, 0) as eng:
+        eng.set_maps(cls, start)
+        for i in range(n_tables):
+            eng.q_set(i, saved_q.reshape(n_tables, -1)[i])
+        eng.set_state(saved_st["s"], saved_st["ep_step"], saved_st["episode"])
+        eng.step_count = saved_t
+        eng.run_fused(rest)
+        got_st, got_q = eng.get_state(), eng.q_get(0, n_tables)
+        assert eng.step_count == first + rest
+    assert np.array_equal(got_q, want_q, equal_nan=True) and np.isfinite(want_q).all()
+    for k in ("s", "ep_step", "episode", "reward", "done", "action"):
+        assert np.array_equal(got_st[k], want_st[k]), k
+    assert np.count_nonzero(want_q) > 100 and want_st["episode"].min() >= 5
+
+
 # ---- explicit batches (CudaQLearning::update_batch) --------------------------------
 
 @pytest.mark.parametrize("mode", [0, 1])
@@ -510,6 +548,27 @@ def test_step_rule_brute_force_against_float_grid(gpu, oracle):
             assert (st["s"][i], st["reward"][i], st["done"][i]) == (y * W + x, np.float32(r), d), (trial, i)
 
 
+def test_step_rule_hand_worked_cell_rewards(gpu):
+    """The hand-worked cases of tests/test_oracle_pins.py (per-cell base rewards, diagonals
+    with cell rewards, both goal modes) through crl_step: literal expectations, no oracle."""
+    from test_oracle_pins import HAND_CASES, HAND_MAP
+    m = HAND_MAP
+    cls, cr = np.array(m["cls"], np.uint8), np.array(m["cr"], np.float32)
+    groups = {}
+    for flags, goal_mode, s, a, want in HAND_CASES:
+        groups.setdefault((flags, goal_mode), []).append((s, a, want))
+    for (flags, goal_mode), cases in groups.items():
+        cfg = gpu.make_config(len(cases), m["W"], m["H"], n_actions=8, map_mode=gpu.MAP_SHARED,
+                              reward_flags=flags, goal_mode=goal_mode, auto_reset=0, trap_reward=-0.75)
+        with gpu.Engine(cfg, 0) as eng:
+            eng.set_maps(cls, np.array([c[0] for c in cases], np.int32), cr if flags else None)
+            eng.step(np.array([c[1] for c in cases], np.int32))
+            st = eng.get_state()
+        for i, (s, a, want) in enumerate(cases):
+            got = (int(st["s"][i]), st["reward"][i], int(st["done"][i]))
+            assert got == (want[0], np.float32(want[1]), want[2]), (flags, goal_mode, s, a, got)
+
+
 def test_full_size_config4(gpu, oracle):
     """The whole 1,048,576-env / 4 GB configuration for its 1000 steps: three
     1024-env slices (first, middle, last) bit-exact against the oracle, and
@@ -537,6 +596,106 @@ def test_full_size_config4(gpu, oracle):
     assert (here < 2).all()
     assert set(np.unique(st["reward"]).tolist()) <= {np.float32(-0.01), np.float32(1.0), np.float32(-1.0)}
     assert (st["ep_step"] < 128).all() and st["episode"].min() >= steps // 128
+
+
+def config5(gpu, n, seed=0):
+    return gpu.make_config(n, 256, 256, n_actions=8, episode_len=1024, lr=0.1, gamma=0.99,
+                           eps_mode=gpu.EPS_EPISODE_LINEAR, eps0=1.0, eps_end=0.05, eps_span=100, seed=seed,
+                           reward_flags=gpu.REWARD_CELLS | gpu.REWARD_BASE_CELLS)
+
+
+def test_config5_shape_untraced_pairs_kernel(gpu, oracle):
+    """Config 5 at its own shape - 256x256 value-noise maps, 8 actions, per-cell
+    rewards, T = 1024, epsilon 1.0 -> 0.05 over 100 episodes - for a few hundred
+    envs and more than two episodes, untraced, so that the kernel the benchmark
+    times runs (folded loop, two lanes per env, move codes from global memory):
+    every table and all state bit-exact against the oracle."""
+    N, steps = 320, 2 * 1024 + 77
+    cls, start, cr = gpu.gen_maps_noise(0, N, 256, 256, 16, 0.25, 0.05, 10.0)
+    cfg = config5(gpu, N)
+    with gpu.Engine(cfg, 0) as eng:
+        eng.set_maps(cls, start, cr)
+        assert eng.fused_kernel_info(steps)["name"] == "k_fused_per_env<8,2,fast,pairs>"
+        eng.run_fused(1024)  # in two launches: the second starts mid-way with trained tables
+        eng.run_fused(steps - 1024)
+        st, q = eng.get_state(), eng.q_get(0, N)
+    Q = np.zeros((N, 256 * 256, 8), np.float32)
+    ost = oracle.new_state(cfg, start)
+    oracle.run(cfg, cls, cr, start, Q, ost, 0, steps)
+    assert_q_close(q.reshape(Q.shape), Q)
+    for k in ("s", "ep_step", "episode", "reward", "done", "action"):
+        assert np.array_equal(st[k], ost[k]), k
+    assert st["episode"].min() >= 2 and np.count_nonzero(Q) > N * 1000
+
+
+def test_full_size_config5(gpu, oracle):
+    """The whole 8192-env / 16 GB configuration for two episodes and a bit: three
+    128-env slices bit-exact against the oracle (tables and state), and
+    size-independent properties over all envs."""
+    from conftest import oracle_run_slice
+    N, W, H, steps = 8192, 256, 256, 2 * 1024 + 100
+    S = W * H
+    cls, start, cr = gpu.gen_maps_noise(0, N, W, H, 16, 0.25, 0.05, 10.0)
+    cfg = config5(gpu, N)
+    slices = [(0, 128), (N // 2 + 5, N // 2 + 5 + 128), (N - 128, N)]
+    with gpu.Engine(cfg, 0) as eng:
+        eng.set_maps(cls, start, cr)
+        info = eng.fused_kernel_info(steps)
+        eng.run_fused(steps)
+        st = eng.get_state()
+        qs = [eng.q_get(lo, hi - lo) for lo, hi in slices]
+    assert info["name"] == "k_fused_per_env<8,2,fast,pairs>"
+    for (lo, hi), q in zip(slices, qs):
+        Q, ost = oracle_run_slice(oracle, cfg, lo, hi, cls[lo:hi], start[lo:hi], 0, steps, cr=cr[lo:hi])
+        assert_q_close(q.reshape(Q.shape), Q)
+        for k in ("s", "ep_step", "episode", "reward", "done", "action"):
+            assert np.array_equal(st[k][lo:hi], ost[k]), (lo, k)
+    env = np.arange(N)
+    assert (cls[env, st["s"]] < 2).all()                      # nobody stands in a wall
+    assert (st["ep_step"] < 1024).all() and (st["episode"] >= 2).all() and (st["action"] < 8).all()
+    assert np.isfinite(st["reward"]).all() and np.abs(st["reward"]).max() < 10.5
+    # an env that has not just restarted got the reward of the cell it stands on
+    # (per-cell base rewards; there are no traps in these maps)
+    moved_on = st["ep_step"] > 0
+    assert np.array_equal(st["reward"][moved_on], cr[env, st["s"]][moved_on])
+    assert ((st["done"] == 1) <= (st["ep_step"] == 0)).all()  # reaching the goal restarts the env
+
+
+def test_large_batches_of_large_per_env_maps(gpu, oracle):
+    """Per-env maps so large that only one or two 64-env waves' worth fit the LDS of
+    a workgroup (the planner has to give up waves, and the plain ticket kernels
+    need more than the default 64 KB): 65,536+ envs, two slices against the oracle."""
+    from conftest import oracle_run_slice
+    for N, W, H, steps in ((65536, 64, 64, 8), (66000, 40, 40, 150), (65536, 48, 48, 70)):
+        cls, start = gpu.gen_maps_bernoulli(4, N, N, W, H, 0.15, 0.02)
+        cfg = gpu.make_config(N, W, H, episode_len=64, eps0=0.15, seed=4)
+        with gpu.Engine(cfg, 0) as eng:
+            eng.set_maps(cls, start)
+            info = eng.fused_kernel_info(steps)
+            assert info["lds_bytes"] <= 160 * 1024
+            eng.run_fused(steps)
+            st = eng.get_state()
+            slices = [(0, 256), (N - 300, N)]
+            qs = [eng.q_get(lo, hi - lo) for lo, hi in slices]
+        for (lo, hi), q in zip(slices, qs):
+            Q, ost = oracle_run_slice(oracle, cfg, lo, hi, cls[lo:hi], start[lo:hi], 0, steps)
+            assert_q_close(q.reshape(Q.shape), Q)
+            for k in ("s", "ep_step", "episode", "reward", "done", "action"):
+                assert np.array_equal(st[k][lo:hi], ost[k]), (N, W, lo, k, info)
+        assert (cls[np.arange(N), st["s"]] < 2).all()
+
+
+def test_full_size_config3_into_the_overflow_regime(gpu, oracle):
+    """65,536 envs on the shared 64x64 table with the configuration's own lr = 0.05
+    for 150 steps: the table overflows on the way (inf / NaN), and every
+    trajectory of the first 4096 envs, the final state of all envs and the table -
+    NaN placement included - equal the oracle's."""
+    N, W, H, steps = 65536, 64, 64, 150
+    cls, start = gpu.gen_maps_bernoulli(0, 1, N, W, H, 0.15)
+    cfg = gpu.make_config(N, W, H, table_mode=gpu.TABLE_SHARED, map_mode=gpu.MAP_SHARED, lr=0.05,
+                          gamma=0.99, eps0=0.2, seed=0)
+    _, q = run_both(gpu, oracle, cfg, cls, start, steps, trace_n=4096)
+    assert not np.isfinite(q).all()
 
 
 @pytest.mark.parametrize("fixture", ["baseline", "reference"])

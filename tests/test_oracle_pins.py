@@ -230,6 +230,61 @@ def test_step_cls_diagonals(oracle, pycrl):
     assert oracle.step_cls(cfg, cls, None, 0, 7)[0] == 0  # UL out of bounds
 
 
+# A 4x3 map holding every class, with per-cell rewards cr[c] = c + 0.5 so that a
+# reward names the cell it was read from.  Expectations are worked by hand from the
+# rule (goal / trap pay on the TARGET cell, anything else on the cell the env stands
+# on after the move when CRL_REWARD_BASE_CELLS is set, else the step reward):
+#      x0  x1  x2  x3
+#  y0  F0  F1  G2  F3
+#  y1  F4  T5  W6  F7
+#  y2  F8  F9  F10 F11
+HAND_MAP = dict(W=4, H=3, cls=[0, 0, 1, 0, 0, 2, 3, 0, 0, 0, 0, 0], cr=[c + 0.5 for c in range(12)])
+# (reward_flags, goal_mode, s, action) -> (s after, reward, hit)
+HAND_CASES = [
+    # per-cell base rewards, goal test on the target cell
+    (3, 0, 1, 1, (2, 2.5, 1)),    # right onto the goal: moves, goal cell pays
+    (3, 0, 1, 2, (1, 5.5, 0)),    # down into the trap: stays, the trap cell pays
+    (3, 0, 7, 3, (7, 7.5, 0)),    # left into the wall: stays, own cell pays
+    (3, 0, 0, 0, (0, 0.5, 0)),    # up out of the grid: stays, own cell pays
+    (3, 0, 0, 1, (1, 1.5, 0)),    # plain move: the cell moved onto pays
+    (3, 0, 9, 4, (9, 9.5, 0)),    # up-right (2,1) is the wall: stays
+    (3, 0, 8, 4, (8, 5.5, 0)),    # up-right (1,1) is the trap: stays, trap pays
+    (3, 0, 7, 7, (2, 2.5, 1)),    # up-left (2,0) is the goal
+    (3, 0, 4, 5, (9, 9.5, 0)),    # down-right (1,2) free
+    (3, 0, 3, 6, (3, 3.5, 0)),    # down-left (2,1) is the wall
+    (3, 0, 11, 5, (11, 11.5, 0)),  # down-right out of the grid
+    (3, 0, 2, 0, (2, 2.5, 0)),    # on the goal, bump: target test does not fire again
+    # goal / trap rewards from the cells only: a plain step pays the step reward
+    (1, 0, 0, 1, (1, -0.01, 0)),
+    (1, 0, 1, 1, (2, 2.5, 1)),
+    (1, 0, 1, 2, (1, 5.5, 0)),
+    (1, 0, 7, 3, (7, -0.01, 0)),
+    (1, 0, 4, 5, (9, -0.01, 0)),
+    # goal test on the resulting cell (src/environment.cu:43): fires again on a bump
+    (3, 1, 2, 0, (2, 2.5, 1)),
+    (3, 1, 2, 2, (2, 2.5, 1)),
+    (3, 1, 1, 2, (1, 5.5, 0)),
+    (3, 1, 1, 1, (2, 2.5, 1)),
+    (3, 1, 0, 1, (1, 1.5, 0)),
+    (3, 1, 7, 7, (2, 2.5, 1)),
+    # class rewards (no cell array): step -0.01, goal 1, trap -0.75
+    (0, 0, 1, 2, (1, -0.75, 0)),
+    (0, 0, 1, 1, (2, 1.0, 1)),
+    (0, 0, 8, 4, (8, -0.75, 0)),
+    (0, 0, 9, 4, (9, -0.01, 0)),
+]
+
+
+def test_step_cls_hand_worked_cell_rewards(oracle, pycrl):
+    m = HAND_MAP
+    cls, cr = np.array(m["cls"], np.uint8), np.array(m["cr"], np.float32)
+    for flags, goal_mode, s, a, want in HAND_CASES:
+        cfg = pycrl.make_config(1, m["W"], m["H"], n_actions=8, reward_flags=flags, goal_mode=goal_mode,
+                                auto_reset=0, trap_reward=-0.75)
+        s2, r, hit = oracle.step_cls(cfg, cls, cr if flags else None, s, a)
+        assert (s2, r, hit) == (want[0], np.float32(want[1]), want[2]), (flags, goal_mode, s, a)
+
+
 # ---- S2 argmax ---------------------------------------------------------------
 
 def test_argmax_lowest_index_on_ties(oracle):
@@ -248,6 +303,32 @@ def test_td_single_sample_zero_table(oracle):
     oracle.lib.orc_td_update_one(oracle._p(q), 4, 1, 2, -0.01, 3, 0, 0.1, 0.99, 0)
     assert q[1 * 4 + 2] == np.float32(np.float32(0.1) * np.float32(-0.01))
     assert np.count_nonzero(q) == 1
+
+
+def test_td_summed_form_single_sample_is_two_roundings(oracle):
+    """One sample on one table through the batch / shared-table form: Q + lr*(target - Q)
+    with the product rounded before the add (the form that sums over duplicates) -
+    equal to the numpy float32 expression, and off the contracted fmaf(lr, target - Q, Q)
+    that the per-env path and nvcc's single-sample update use by no more than that one
+    extra rounding (half an ulp of the product, plus the final rounding)."""
+    rng = np.random.default_rng(3)
+    f32 = np.float32
+    lr, gamma = f32(0.1), f32(0.99)
+    differ = 0
+    for _ in range(2000):
+        q0, r, m = (f32(v) for v in rng.normal(0, 1, 3))
+        Q = np.zeros((2, 4), f32)
+        Q[0, 1], Q[1] = q0, [m, m - f32(1), m - f32(2), m - f32(3)]
+        oracle.td_update_batch(Q, 2, 4, [0], [1], [r], [1], [0], float(lr), float(gamma), 0)
+        target = f32(np.float64(gamma) * np.float64(m) + np.float64(r))  # fmaf(gamma, m, r): one rounding
+        prod = f32(lr * f32(target - q0))
+        want = f32(q0 + prod)
+        assert Q[0, 1] == want
+        fused = f32(oracle.lib.orc_td_value(q0, r, m, lr, gamma))
+        bound = 0.5 * float(np.spacing(np.abs(prod))) + float(np.spacing(np.abs(want)))
+        assert abs(float(fused) - float(want)) <= bound
+        differ += fused != want
+    assert 0 < differ < 1500  # the two forms do differ on a fair share of inputs
 
 
 def test_td_self_loop_geometric_series(oracle):
