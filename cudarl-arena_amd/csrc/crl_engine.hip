@@ -10,6 +10,7 @@
 #include <cstring>
 #include <exception>
 #include <memory>
+#include <mutex>
 #include <new>
 #include <string>
 #include <vector>
@@ -79,6 +80,37 @@ struct DevBuf {
   DevBuf& operator=(const DevBuf&) = delete;
 };
 
+// Scratch of crl_run_fused_noalloc: one array per GPU, part of the loaded code
+// object, so the entry point never allocates.  Layout: 256 bytes of ticket
+// counters, then the hand-off cells of the ordered reduction.  The array's name
+// is a host-side stand-in, not a device address: host code only ever uses the
+// address hipGetSymbolAddress returned for the device at hand.
+constexpr size_t kScratchTicketBytes = 256;
+constexpr size_t kScratchHandoffBytes = (size_t)8 << 20;
+constexpr size_t kScratchBytes = kScratchTicketBytes + kScratchHandoffBytes;
+static __device__ __align__(256) unsigned char scratch[kScratchBytes];
+
+constexpr int kMaxDevices = 64;
+std::mutex g_scratch_lock;
+unsigned char* g_scratch_ptr[kMaxDevices] = {};
+
+// Address of `device`'s copy of the scratch array; looked up once per device, with
+// that device current.  Called from crl_create, so that crl_run_fused_noalloc
+// finds it there.
+int scratch_of_device(int device, unsigned char** out) {
+  if (device < 0 || device >= kMaxDevices) return fail(CRL_E_ARG, "device %d: at most %d devices", device, kMaxDevices);
+  std::lock_guard<std::mutex> hold(g_scratch_lock);
+  if (!g_scratch_ptr[device]) {
+    HIP_TRY(hipSetDevice(device));
+    void* p = nullptr;
+    HIP_TRY(hipGetSymbolAddress(&p, HIP_SYMBOL(scratch)));
+    if (!p) return fail(CRL_E_DEVICE, "hipGetSymbolAddress returned no address for the scratch array");
+    g_scratch_ptr[device] = static_cast<unsigned char*>(p);
+  }
+  *out = g_scratch_ptr[device];
+  return CRL_OK;
+}
+
 }  // namespace
 
 struct crl_engine {
@@ -94,6 +126,13 @@ struct crl_engine {
   int fused_variant = 0;   // 0 = automatic, 1 = plain, 2 = hybrid (when it fits)
   DevBuf<unsigned> ticket;
   bool hybrid_opt_in = false;
+  // the scratch the call in progress works with: the engine's own allocations
+  // (crl_run_fused, crl_update, crl_td_update) or the device's static array
+  // (crl_run_fused_noalloc)
+  bool no_alloc = false;
+  unsigned char* static_scratch = nullptr;
+  unsigned* tk = nullptr;  // ticket counters {next ticket, envs on HBM tables, envs on LDS tables}
+  uint2* ho = nullptr;     // hand-off cells of the ordered reduction
 
   DevBuf<int32_t> s, ep_step, episode, start, act;
   DevBuf<float> reward;
@@ -391,9 +430,9 @@ void launch_fused_a(const crl_engine* e, const FusedPlan& p, uint64_t t0, int n)
   const crl::Ptrs P = e->ptrs();
   if (p.tickets) {
     // (tickets dealt by position use no counter; the kernel itself notes who did how much)
-    if (!p.fixed) hipLaunchKernelGGL(crl::k_fill_u32, dim3(1), dim3(64), 0, e->stream, e->ticket.p, 0u, 3);
+    if (!p.fixed) hipLaunchKernelGGL(crl::k_fill_u32, dim3(1), dim3(64), 0, e->stream, e->tk, 0u, 3);
     const dim3 g(p.grid), b(p.block);
-    unsigned* tk = e->ticket.p;
+    unsigned* tk = e->tk;
 #define CRL_LAUNCH_TICKETS(MODE, LDSW, MOVES)                                                       \
   hipLaunchKernelGGL((crl::k_fused_tickets<A, MODE, LDSW, MOVES>), g, b, p.lds, e->stream, R, P, t0, n, \
                      tk, p.tab_stride, p.fixed ? 1 : 0, p.pair ? 1 : 0)
@@ -481,15 +520,23 @@ int opt_in_lds(crl_engine* e) {
 
 int ensure_handoff(crl_engine* e, const crl::ReduceGeom& G) {
   const size_t recs = handoff_records(G);
-  hipError_t h = e->handoff.ensure(recs);
-  if (h != hipSuccess) return fail(CRL_E_ALLOC, "hand-off buffer allocation failed: %s", hipGetErrorString(h));
+  if (e->no_alloc) {
+    if (recs * sizeof(uint2) > kScratchHandoffBytes)
+      return fail(CRL_E_RANGE, "the ordered reduction of this engine needs %zu bytes of hand-off cells, "
+                  "the static scratch of crl_run_fused_noalloc holds %zu", recs * sizeof(uint2), kScratchHandoffBytes);
+    e->ho = reinterpret_cast<uint2*>(e->static_scratch + kScratchTicketBytes);
+  } else {
+    hipError_t h = e->handoff.ensure(recs);
+    if (h != hipSuccess) return fail(CRL_E_ALLOC, "hand-off buffer allocation failed: %s", hipGetErrorString(h));
+    e->ho = e->handoff.p;
+  }
   return opt_in_lds(e);
 }
 
 int reduce_owners(crl_engine* e, const crl::ReduceGeom& G, float* Q, const int32_t* key,
                   const float* delta, int n) {
   hipLaunchKernelGGL(crl::k_reduce_owners, dim3(1 << G.own_shift), dim3(256), kOwnersLds, e->stream, G,
-                     Q, key, delta, n, e->handoff.p);
+                     Q, key, delta, n, e->ho);
   HIP_TRY(hipGetLastError());
   return CRL_OK;
 }
@@ -497,6 +544,7 @@ int reduce_owners(crl_engine* e, const crl::ReduceGeom& G, float* Q, const int32
 // Q[k] += ordered sum of delta[i] with key[i] == k, for n samples on one table
 int reduce_apply(crl_engine* e, float* Q, const int32_t* key, const float* delta, int n) {
   const crl::ReduceGeom G = reduce_geom(e, n);
+  e->no_alloc = false;  // crl_update / crl_td_update: the engine's own hand-off buffer
   if (!reduce_fast(e, G)) {
     const int grid = (int)((e->K + crl::kOwnKeys - 1) / crl::kOwnKeys);
     hipLaunchKernelGGL(crl::k_reduce_scan, dim3(grid), dim3(256), 0, e->stream, Q, (int)e->K, key,
@@ -507,7 +555,7 @@ int reduce_apply(crl_engine* e, float* Q, const int32_t* key, const float* delta
   int rc = ensure_handoff(e, G);
   if (rc) return rc;
   hipLaunchKernelGGL(crl::k_reduce_blocks, dim3(G.n_blocks), dim3(crl::kBlockSamples),
-                     sizeof(crl::ReduceLds), e->stream, G, key, delta, n, e->handoff.p);
+                     sizeof(crl::ReduceLds), e->stream, G, key, delta, n, e->ho);
   HIP_TRY(hipGetLastError());
   return reduce_owners(e, G, Q, key, delta, n);
 }
@@ -520,10 +568,10 @@ void launch_shared_act(crl_engine* e, bool reduce, const crl::ReduceGeom& G, uin
   const size_t lds = (reduce ? sizeof(crl::ReduceLds) : 0) + (MAP == 1 ? (size_t)e->map_words * 4 : 0);
   if (reduce)
     hipLaunchKernelGGL((crl::k_shared_act<A, MAP, true>), dim3(grid), dim3(block), lds, e->stream, R, P,
-                       t, trace_row, e->key.p, e->delta.p, G, e->handoff.p);
+                       t, trace_row, e->key.p, e->delta.p, G, e->ho);
   else
     hipLaunchKernelGGL((crl::k_shared_act<A, MAP, false>), dim3(grid), dim3(block), lds, e->stream, R,
-                       P, t, trace_row, e->key.p, e->delta.p, G, e->handoff.p);
+                       P, t, trace_row, e->key.p, e->delta.p, G, e->ho);
 }
 
 // one shared-table step: act (select + move + delta + block sums), then the key owners
@@ -614,6 +662,8 @@ int upload_maps(crl_engine* e) {
   HIP_TRY(hipStreamSynchronize(e->stream));
   return CRL_OK;
 }
+
+int opt_in_ticket_kernels(crl_engine* e);
 
 int create_engine(const crl_config* cfg, int device, crl_engine** out) {
   if (!out) return fail(CRL_E_ARG, "out is null");
@@ -708,6 +758,11 @@ int create_engine(const crl_config* cfg, int device, crl_engine** out) {
                           hipMemcpyHostToDevice, e->stream)) != hipSuccess)
     return bail(h, "upload cell rewards");
   if ((h = hipStreamSynchronize(e->stream)) != hipSuccess) return bail(h, "sync");
+  // set-up that crl_run_fused_noalloc must not have left to do: this device's copy
+  // of the scratch array, and the kernels that may use the whole LDS
+  rc = scratch_of_device(device, &e->static_scratch);
+  if (rc == CRL_OK) rc = cfg->table_mode == CRL_TABLE_SHARED ? opt_in_lds(e) : opt_in_ticket_kernels(e);
+  if (rc != CRL_OK) return rc;
   *out = own.release();
   return CRL_OK;
 }
@@ -777,6 +832,77 @@ int set_cell(crl_engine* e, int32_t map_index, int32_t cell, int32_t cell_class,
   return CRL_OK;
 }
 
+// every ticket-kernel instantiation launch_fused_a can pick may use the whole LDS:
+// the plain ones, too, ask for more than the default 64 KB when large per-env
+// maps share a workgroup
+int opt_in_ticket_kernels(crl_engine* e) {
+  if (e->hybrid_opt_in) return CRL_OK;
+  const void* fns[] = {
+#define CRL_TICKET_KERNELS(A)                                                          \
+  reinterpret_cast<const void*>(&crl::k_fused_tickets<A, 0, false, false>),            \
+      reinterpret_cast<const void*>(&crl::k_fused_tickets<A, 1, false, false>),        \
+      reinterpret_cast<const void*>(&crl::k_fused_tickets<A, 2, false, false>),        \
+      reinterpret_cast<const void*>(&crl::k_fused_tickets<A, 0, true, false>),         \
+      reinterpret_cast<const void*>(&crl::k_fused_tickets<A, 1, true, false>),         \
+      reinterpret_cast<const void*>(&crl::k_fused_tickets<A, 1, false, true>),         \
+      reinterpret_cast<const void*>(&crl::k_fused_tickets<A, 2, false, true>)
+      CRL_TICKET_KERNELS(4), CRL_TICKET_KERNELS(8)
+#undef CRL_TICKET_KERNELS
+  };
+  for (const void* fn : fns)
+    HIP_TRY(hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, (int)kLdsPerWorkgroup));
+  e->hybrid_opt_in = true;
+  return CRL_OK;
+}
+
+// crl_run_fused and its allocation-free variant: with `no_alloc` the ticket
+// counters and the hand-off cells live in the device's static scratch array and
+// nothing below allocates or frees
+int run_fused(crl_engine* e, int32_t n_steps, bool no_alloc) {
+  int rc = check_engine(e);
+  if (rc) return rc;
+  if (n_steps < 0) return fail(CRL_E_ARG, "negative step count");
+  if (n_steps == 0) return CRL_OK;
+  if (no_alloc && !e->static_scratch) return fail(CRL_E_STATE, "the device's scratch array was not found at crl_create");
+  e->no_alloc = no_alloc;
+  if (e->cfg.table_mode == CRL_TABLE_PER_ENV) {
+    const FusedPlan p = plan_fused(e, n_steps);
+    if (p.lds > kLdsPerWorkgroup)
+      return fail(CRL_E_STATE, "launch plan %s needs %zu bytes of LDS per workgroup, the device has %zu",
+                  p.name, p.lds, kLdsPerWorkgroup);
+    if (p.tickets) {
+      if (no_alloc) {
+        e->tk = reinterpret_cast<unsigned*>(e->static_scratch);
+      } else {
+        if (e->ticket.ensure(3) != hipSuccess) return fail(CRL_E_ALLOC, "ticket counter allocation failed");
+        e->tk = e->ticket.p;
+      }
+      rc = opt_in_ticket_kernels(e);  // done at crl_create; a no-op here
+      if (rc) return rc;
+    }
+    if (e->A == 4)
+      launch_fused_a<4>(e, p, e->t, n_steps);
+    else
+      launch_fused_a<8>(e, p, e->t, n_steps);
+    HIP_TRY(hipGetLastError());
+    if (e->trace_n > 0) {
+      const long long c = (long long)e->trace_cursor + n_steps;
+      e->trace_cursor = c > e->trace_cap ? e->trace_cap : (int)c;
+    }
+  } else {
+    for (int k = 0; k < n_steps; ++k) {
+      rc = shared_step(e, e->t + (uint64_t)k, e->trace_cursor);
+      if (rc) return rc;
+      if (e->trace_n > 0 && e->trace_cursor < e->trace_cap) e->trace_cursor += 1;
+    }
+  }
+  e->no_alloc = false;
+  e->t += (uint64_t)n_steps;
+  e->have_transition = false;
+  e->have_actions = false;
+  return CRL_OK;
+}
+
 }  // namespace
 
 extern "C" {
@@ -820,7 +946,7 @@ int crl_set_resident_envs(crl_engine* e, int32_t n_envs) {
 
 int crl_set_fused_variant(crl_engine* e, int32_t variant) {
   if (!e) return fail(CRL_E_ARG, "null engine");
-  if (variant < 0 || variant > 2) return fail(CRL_E_ARG, "variant must be 0 (automatic), 1 (plain) or 2 (hybrid)");
+  if (variant < 0 || variant > 2) return fail(CRL_E_ARG, "variant must be 0 (automatic), 1 or 2");
   e->fused_variant = variant;
   return CRL_OK;
 }
@@ -829,8 +955,8 @@ int crl_get_fused_split(crl_engine* e, uint32_t* hbm_envs, uint32_t* lds_envs) {
   int rc = check_engine(e);
   if (rc) return rc;
   unsigned v[3] = {0, 0, 0};
-  if (e->ticket.p) {
-    HIP_TRY(hipMemcpyAsync(v, e->ticket.p, sizeof v, hipMemcpyDeviceToHost, e->stream));
+  if (e->tk) {
+    HIP_TRY(hipMemcpyAsync(v, e->tk, sizeof v, hipMemcpyDeviceToHost, e->stream));
     HIP_TRY(hipStreamSynchronize(e->stream));
   }
   if (hbm_envs) *hbm_envs = v[1];
@@ -974,59 +1100,9 @@ int crl_td_update(crl_engine* e, int32_t table, int32_t n, const int32_t* s, con
   return reduce_apply(e, Q, e->key.p, e->delta.p, n);
 }
 
-int crl_run_fused(crl_engine* e, int32_t n_steps) {
-  int rc = check_engine(e);
-  if (rc) return rc;
-  if (n_steps < 0) return fail(CRL_E_ARG, "negative step count");
-  if (n_steps == 0) return CRL_OK;
-  if (e->cfg.table_mode == CRL_TABLE_PER_ENV) {
-    const FusedPlan p = plan_fused(e, n_steps);
-    if (p.lds > kLdsPerWorkgroup)
-      return fail(CRL_E_STATE, "launch plan %s needs %zu bytes of LDS per workgroup, the device has %zu",
-                  p.name, p.lds, kLdsPerWorkgroup);
-    if (p.tickets) {
-      if (e->ticket.ensure(3) != hipSuccess) return fail(CRL_E_ALLOC, "ticket counter allocation failed");
-      if (!e->hybrid_opt_in) {
-        // every instantiation launch_fused_a can pick: the plain ones, too, ask for
-        // more than the default 64 KB when large per-env maps share a workgroup
-        const void* fns[] = {
-#define CRL_TICKET_KERNELS(A)                                                          \
-  reinterpret_cast<const void*>(&crl::k_fused_tickets<A, 0, false, false>),            \
-      reinterpret_cast<const void*>(&crl::k_fused_tickets<A, 1, false, false>),        \
-      reinterpret_cast<const void*>(&crl::k_fused_tickets<A, 2, false, false>),        \
-      reinterpret_cast<const void*>(&crl::k_fused_tickets<A, 0, true, false>),         \
-      reinterpret_cast<const void*>(&crl::k_fused_tickets<A, 1, true, false>),         \
-      reinterpret_cast<const void*>(&crl::k_fused_tickets<A, 1, false, true>),         \
-      reinterpret_cast<const void*>(&crl::k_fused_tickets<A, 2, false, true>)
-            CRL_TICKET_KERNELS(4), CRL_TICKET_KERNELS(8)
-#undef CRL_TICKET_KERNELS
-        };
-        for (const void* fn : fns)
-          HIP_TRY(hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, (int)kLdsPerWorkgroup));
-        e->hybrid_opt_in = true;
-      }
-    }
-    if (e->A == 4)
-      launch_fused_a<4>(e, p, e->t, n_steps);
-    else
-      launch_fused_a<8>(e, p, e->t, n_steps);
-    HIP_TRY(hipGetLastError());
-    if (e->trace_n > 0) {
-      const long long c = (long long)e->trace_cursor + n_steps;
-      e->trace_cursor = c > e->trace_cap ? e->trace_cap : (int)c;
-    }
-  } else {
-    for (int k = 0; k < n_steps; ++k) {
-      rc = shared_step(e, e->t + (uint64_t)k, e->trace_cursor);
-      if (rc) return rc;
-      if (e->trace_n > 0 && e->trace_cursor < e->trace_cap) e->trace_cursor += 1;
-    }
-  }
-  e->t += (uint64_t)n_steps;
-  e->have_transition = false;
-  e->have_actions = false;
-  return CRL_OK;
-}
+int crl_run_fused(crl_engine* e, int32_t n_steps) { return run_fused(e, n_steps, false); }
+
+int crl_run_fused_noalloc(crl_engine* e, int32_t n_steps) { return run_fused(e, n_steps, true); }
 
 int crl_get_state(crl_engine* e, int32_t* s, float* reward, uint8_t* done, uint8_t* action,
                   int32_t* ep_step, int32_t* episode) {

@@ -83,7 +83,7 @@ _lib = None
 EXPORTS = [
     "crl_last_error", "crl_version", "crl_device_count", "crl_create", "crl_destroy",
     "crl_set_stream", "crl_sync", "crl_set_resident_envs", "crl_set_fused_variant", "crl_get_fused_split", "crl_set_maps", "crl_set_cell", "crl_classify_grid", "crl_reset",
-    "crl_step", "crl_select", "crl_update", "crl_td_update", "crl_run_fused", "crl_get_state",
+    "crl_step", "crl_select", "crl_update", "crl_td_update", "crl_run_fused", "crl_run_fused_noalloc", "crl_get_state",
     "crl_set_state", "crl_get_episode_stats", "crl_get_step_count", "crl_set_step_count", "crl_q_get", "crl_q_set",
     "crl_q_get_range", "crl_set_trace", "crl_get_trace", "crl_set_exploration_stream",
     "crl_device_ptr", "crl_fused_kernel_info", "crl_fused_plan_for_config", "crl_philox4x32_10", "crl_explore_draw",
@@ -119,6 +119,7 @@ def load():
     lib.crl_update.argtypes = [vp]
     lib.crl_td_update.argtypes = [vp, i32, i32, vp, vp, vp, vp, vp]
     lib.crl_run_fused.argtypes = [vp, i32]
+    lib.crl_run_fused_noalloc.argtypes = [vp, i32]
     lib.crl_get_state.argtypes = [vp, vp, vp, vp, vp, vp, vp]
     lib.crl_set_state.argtypes = [vp, vp, vp, vp]
     lib.crl_get_episode_stats.argtypes = [vp, vp, vp, vp, vp]
@@ -274,6 +275,9 @@ class Engine:
 
     def run_fused(self, n_steps):
         _check(self.lib.crl_run_fused(self.h, n_steps))
+
+    def run_fused_noalloc(self, n_steps):
+        _check(self.lib.crl_run_fused_noalloc(self.h, n_steps))
 
     def set_resident_envs(self, n):
         _check(self.lib.crl_set_resident_envs(self.h, n))

@@ -194,6 +194,19 @@ int crl_td_update(crl_engine* e, int32_t table, int32_t n, const int32_t* s, con
  * crl_select; crl_step(NULL); crl_update. */
 int crl_run_fused(crl_engine* e, int32_t n_steps);
 
+/* crl_run_fused for callers that cannot allocate device memory (work recorded
+ * under HIP graph capture, tight serving loops, harnesses that forbid
+ * hipMalloc): no counterpart in the reference.  Same results as crl_run_fused,
+ * but its scratch - the ticket counters of the per-env kernels, the hand-off
+ * cells of the shared table's ordered reduction - lives in a static device
+ * array of 8 MB + 256 bytes that each GPU the library runs on holds until the
+ * process ends, and the call allocates and frees nothing (device or host).
+ * CRL_E_RANGE if the engine's reduction needs more hand-off cells than the
+ * array holds (65,536 envs on a 64x64x4 table need 4 MB).  All engines on one
+ * GPU share that GPU's array: calls that overlap in time on one GPU (different
+ * streams or threads) race; calls in stream order do not. */
+int crl_run_fused_noalloc(crl_engine* e, int32_t n_steps);
+
 /* Environment getters (src/environment.h:26-37) for all envs; any pointer may
  * be NULL.  s = cell the env acts from next, reward/done/action = last step. */
 int crl_get_state(crl_engine* e, int32_t* s, float* reward, uint8_t* done, uint8_t* action,
