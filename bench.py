@@ -51,7 +51,7 @@ WORKLOADS = {
                      "table 4096x4, ordered reduction, 1000 steps"),
     # traffic: HBM bytes per env-step from rocprofv3 FETCH_SIZE x2.000 + WRITE_SIZE x1.000
     # (profiles/k_fused_tickets_c4.md), valid for the default launch only
-    "c4": dict(n=1 << 20, launch_steps=1000, bytes=42.25, traffic=30.8,
+    "c4": dict(n=1 << 20, launch_steps=1000, bytes=42.25, traffic=29.8,
                name="c4: 1048576 envs 16x16, per-env tables 256x4 (4 GB), traps, eps 0.1, T=128, 1000 steps"),
     "c5": dict(n=8192, launch_steps=1024, bytes=70.0, traffic=None,
                name="c5: 8192 envs 256x256, 8 actions, per-env tables 65536x8 (16 GB), cell rewards, "
@@ -147,12 +147,20 @@ def time_gpu(key, reps, warm_reps, launch_steps=None, n_override=None, resident=
         st = eng.get_state()
         split = eng.fused_split()
         q_probe = eng.q_get(0)
+        phases = None
+        if variant == 2 and cfg.table_mode == pycrl.TABLE_SHARED and info["name"].startswith("k_shared_persist"):
+            # clocks of the LAST launch, first workgroup; scaled to that launch's measured time
+            clk = eng.persist_clocks()[0].astype(float)
+            names = ("wait_for_owners", "act", "block_sums", "drain_publish", "wait_for_blocks", "cells_to_tile",
+                     "tile_sums_publish", "loop")
+            us = rep_ms[-1] * 1e3 / per
+            phases = {k: us * c / clk.sum() for k, c in zip(names, clk)}
     dev_ms = sum(rep_ms)
     secs = max(wall, dev_ms * 1e-3)
     return dict(n=n, launch_steps=per, reps=reps, env_steps=n * per * reps, steps_per_s=n * per * reps / secs,
                 ms_per_rep=secs * 1e3 / reps, device_ms=dev_ms, rep_ms=rep_ms, wall_s=wall, info=info,
                 split=split, episodes_min=int(st["episode"].min()), bytes_per_step=wl["bytes"],
-                table_finite=bool(np.isfinite(q_probe).all()))
+                table_finite=bool(np.isfinite(q_probe).all()), phases=phases)
 
 
 def _cpu_model():
@@ -253,7 +261,10 @@ def cpu_baseline(key, full_n):
 
 def side_figure(key, reps, warm, launch_steps=None):
     r = time_gpu(key, reps, warm, launch_steps)
-    return {"workload": WORKLOADS[key]["name"], "value": r["steps_per_s"], "unit": "env-steps/s",
+    name = WORKLOADS[key]["name"]
+    if launch_steps:
+        name = name.rsplit(",", 1)[0] + ", %d steps per launch" % launch_steps
+    return {"workload": name, "value": r["steps_per_s"], "unit": "env-steps/s",
             "n_envs": r["n"], "steps_per_launch": r["launch_steps"], "launches_timed": reps,
             "us_per_env_step_round": r["device_ms"] * 1e3 / (reps * r["launch_steps"]),
             "median_launch_ms": statistics.median(r["rep_ms"]), "kernel": r["info"]["name"],
@@ -275,6 +286,8 @@ def main():
     ap.add_argument("--variant", type=int, default=0, help="fused kernel: 0 automatic, 1 plain, 2 hybrid")
     ap.add_argument("--probe-copy", type=int, default=0, metavar="MIB",
                     help="only run one plain copy kernel of this many MiB (calibrates rocprofv3 counters)")
+    ap.add_argument("--probe-barrier", action="store_true",
+                    help="only measure barriers over co-resident workgroups built from device-scope loads and stores")
     ap.add_argument("--no-cpu", action="store_true", help="skip the cpu_baseline leg")
     ap.add_argument("--no-also", action="store_true", help="skip the side measurements of the other configs")
     args = ap.parse_args()
@@ -290,6 +303,11 @@ def main():
     if args.probe_copy:
         pycrl._check(lib.crl_probe_copy(args.probe_copy << 20, 3))
         print(json.dumps({"probe_copy_bytes_per_launch": args.probe_copy << 20, "launches": 3}))
+        return
+    if args.probe_barrier:
+        names = {0: "packed flags, everybody polls all", 1: "one flag per 128-byte line", 2: "tree, one reader per word"}
+        print(json.dumps({"ns_per_barrier": {names[p]: {str(n): pycrl.probe_barrier(p, n, 2000) for n in (8, 64, 256)}
+                                             for p in (0, 1, 2)}, "rounds": 2000, "block": 256}))
         return
     key = args.workload
     wl = WORKLOADS[key]
@@ -329,6 +347,8 @@ def main():
                      "algorithmic_bytes_per_launch": bytes_per_launch,
                      "kernel_ms_per_launch": avg_launch_ms},
     }
+    if g["phases"]:
+        out["config"]["us_per_step_by_phase"] = g["phases"]
     if wl.get("traffic") and default_shape:
         # bytes past the L2 per launch, measured in separate rocprofv3 --pmc runs of this
         # same command (profiles/), not in this run

@@ -18,6 +18,7 @@
 #include "../../include/crl.h"
 #include "crl_host.h"
 #include "crl_kernels.h"
+#include "crl_persist.h"
 
 namespace {
 
@@ -81,11 +82,13 @@ struct DevBuf {
 };
 
 // Scratch of crl_run_fused_noalloc: one array per GPU, part of the loaded code
-// object, so the entry point never allocates.  Layout: 256 bytes of ticket
-// counters, then the hand-off cells of the ordered reduction.  The array's name
+// object, so the entry point never allocates.  Layout: 4 KB of counters (ticket
+// counters at 0, the one-launch shared-table kernel's step flags at 1 KB and its
+// give-up word at 3 KB), then the hand-off cells of the ordered reduction.  The array's name
 // is a host-side stand-in, not a device address: host code only ever uses the
 // address hipGetSymbolAddress returned for the device at hand.
-constexpr size_t kScratchTicketBytes = 256;
+constexpr size_t kScratchTicketBytes = 4096;
+constexpr size_t kScratchFlagsAt = 1024, kScratchErrAt = 3072;
 constexpr size_t kScratchHandoffBytes = (size_t)8 << 20;
 constexpr size_t kScratchBytes = kScratchTicketBytes + kScratchHandoffBytes;
 static __device__ __align__(256) unsigned char scratch[kScratchBytes];
@@ -133,6 +136,12 @@ struct crl_engine {
   unsigned char* static_scratch = nullptr;
   unsigned* tk = nullptr;  // ticket counters {next ticket, envs on HBM tables, envs on LDS tables}
   uint2* ho = nullptr;     // hand-off cells of the ordered reduction
+  // one-launch shared-table kernel: step flags + give-up word, and whether a launch
+  // has not been checked for having given up yet
+  DevBuf<unsigned> pflags;
+  unsigned* perr = nullptr;
+  bool persist_unchecked = false;
+  bool persist_refused = false;  // the device refused the co-resident launch once: not tried again
 
   DevBuf<int32_t> s, ep_step, episode, start, act;
   DevBuf<float> reward;
@@ -275,6 +284,7 @@ struct FusedPlan {
 };
 
 constexpr size_t kLdsPerWorkgroup = 160 * 1024;  // gfx950
+constexpr size_t kPersistStaticLds = 1024;      // static LDS of the one-launch shared-table kernel, rounded up
 
 // Launches shorter than this do not repay moving whole tables into LDS and back
 // (1M envs of config 4, steps per launch -> env-steps/s, plain / hybrid:
@@ -514,12 +524,16 @@ int opt_in_lds(crl_engine* e) {
   HIP_TRY(allow_lds(crl::k_shared_act<4, 2, true>, act));
   HIP_TRY(allow_lds(crl::k_shared_act<8, 1, true>, act));
   HIP_TRY(allow_lds(crl::k_shared_act<8, 2, true>, act));
+  HIP_TRY(allow_lds(crl::k_shared_persist<4, 1>, act - kPersistStaticLds));
+  HIP_TRY(allow_lds(crl::k_shared_persist<4, 2>, act - kPersistStaticLds));
+  HIP_TRY(allow_lds(crl::k_shared_persist<8, 1>, act - kPersistStaticLds));
+  HIP_TRY(allow_lds(crl::k_shared_persist<8, 2>, act - kPersistStaticLds));
   e->lds_opt_in = true;
   return CRL_OK;
 }
 
 int ensure_handoff(crl_engine* e, const crl::ReduceGeom& G) {
-  const size_t recs = handoff_records(G);
+  const size_t recs = handoff_records(G);  // (G.n_blocks: blocks, or workgroups of the one-launch kernel)
   if (e->no_alloc) {
     if (recs * sizeof(uint2) > kScratchHandoffBytes)
       return fail(CRL_E_RANGE, "the ordered reduction of this engine needs %zu bytes of hand-off cells, "
@@ -605,6 +619,109 @@ int shared_step(crl_engine* e, uint64_t t, int trace_row) {
   hipLaunchKernelGGL(crl::k_reduce_scan, dim3(grid), dim3(256), 0, e->stream, e->Q.p, (int)e->K,
                      e->key.p, e->delta.p, e->N);
   HIP_TRY(hipGetLastError());
+  return CRL_OK;
+}
+
+// ---- shared table: all steps of a call in one launch ---------------------------------
+
+struct PersistPlan {  // (kPersistStaticLds: the kernel's own static LDS, rounded up)
+  bool ok;
+  int grid;
+  bool lds_map;
+  size_t lds;
+  crl::ReduceGeom G;
+};
+
+// The one-launch kernel needs every workgroup resident at once (one per compute
+// unit), the dense LDS table of the block pass and one tile of the owners' pass.
+PersistPlan plan_persist(const crl_engine* e, int n_steps) {
+  PersistPlan p{};
+  // Only on request: measured on 65,536 envs / 64x64x4 it takes 16 us per step against the
+  // 12 us of two launches per step - a barrier over 256 workgroups through memory costs
+  // 2.5 to 3 us however the flags are laid out, a kernel boundary 1.6 us.
+  if (e->cfg.table_mode != CRL_TABLE_SHARED || e->fused_variant != 2 || e->persist_refused) return p;
+  const int n_blocks = (e->N + crl::kBlockSamples - 1) / crl::kBlockSamples;
+  p.G = reduce_geom(e, e->N);
+  const int n_own = 1 << p.G.own_shift;
+  p.grid = std::max(n_blocks, n_own);
+  if (e->K > (size_t)crl::kDenseKeys || p.grid > crl::kPersistMaxGroups || p.grid > kComputeUnits) return p;
+  p.G.n_blocks = p.grid;  // workgroups without envs hand over empty cells
+  const size_t map_bytes = (size_t)e->map_words * 4;
+  p.lds_map = e->cfg.map_mode == CRL_MAP_SHARED && crl::kPersistReduceLds + map_bytes <= kLdsPerWorkgroup - kPersistStaticLds;
+  p.lds = crl::kPersistReduceLds + (p.lds_map ? map_bytes : 0);
+  p.ok = true;
+  return p;
+}
+
+template <int A, int MAP>
+hipError_t launch_persist_kernel(crl_engine* e, const PersistPlan& p, int n_steps, unsigned* flags) {
+  crl::Rules R = e->rules();
+  crl::Ptrs P = e->ptrs();
+  uint64_t t0 = e->t;
+  int n = n_steps, trace_row0 = e->trace_cursor;
+  int32_t* key = e->key.p;
+  float* delta = e->delta.p;
+  crl::ReduceGeom G = p.G;
+  uint2* handoff = e->ho;
+  unsigned* err = e->perr;
+  void* args[] = {&R, &P, &t0, &n, &trace_row0, &key, &delta, &G, &handoff, &flags, &err};
+  // a cooperative launch is refused unless all workgroups can be resident together,
+  // which the kernel's waits rely on
+  return hipLaunchCooperativeKernel(reinterpret_cast<const void*>(&crl::k_shared_persist<A, MAP>), dim3(p.grid),
+                                    dim3(256), args, (unsigned)p.lds, e->stream);
+}
+
+// -> CRL_OK and *launched = true, or *launched = false when the caller should take
+// the two-launches-per-step path instead
+int run_persist(crl_engine* e, int n_steps, bool* launched) {
+  *launched = false;
+  const PersistPlan p = plan_persist(e, n_steps);
+  if (!p.ok) return CRL_OK;
+  unsigned* flags;
+  if (e->no_alloc) {
+    flags = reinterpret_cast<unsigned*>(e->static_scratch + kScratchFlagsAt);
+    e->perr = reinterpret_cast<unsigned*>(e->static_scratch + kScratchErrAt);
+  } else {
+    if (e->pflags.ensure(2 * crl::kPersistMaxGroups + 64) != hipSuccess)
+      return fail(CRL_E_ALLOC, "flag allocation failed");
+    flags = e->pflags.p;
+    e->perr = e->pflags.p + 2 * crl::kPersistMaxGroups;
+  }
+  int rc = ensure_handoff(e, p.G);
+  if (rc) return rc;
+  // flags and the give-up word start at zero (the word follows the flags in both layouts'
+  // fill: two fills keep the static layout's gap untouched)
+  hipLaunchKernelGGL(crl::k_fill_u32, dim3(2), dim3(256), 0, e->stream, flags, 0u, 2 * crl::kPersistMaxGroups);
+  hipLaunchKernelGGL(crl::k_fill_u32, dim3(1), dim3(64), 0, e->stream, e->perr, 0u, 1);
+  hipError_t h;
+  if (e->A == 4)
+    h = p.lds_map ? launch_persist_kernel<4, 1>(e, p, n_steps, flags) : launch_persist_kernel<4, 2>(e, p, n_steps, flags);
+  else
+    h = p.lds_map ? launch_persist_kernel<8, 1>(e, p, n_steps, flags) : launch_persist_kernel<8, 2>(e, p, n_steps, flags);
+  if (h != hipSuccess) {
+    (void)hipGetLastError();  // not resident all at once on this device: never mind, two launches per step
+    e->persist_refused = true;
+    return CRL_OK;
+  }
+  e->persist_unchecked = true;
+  if (e->trace_n > 0) {
+    const long long c = (long long)e->trace_cursor + n_steps;
+    e->trace_cursor = c > e->trace_cap ? e->trace_cap : (int)c;
+  }
+  *launched = true;
+  return CRL_OK;
+}
+
+// After a synchronisation: did a one-launch kernel give up waiting for its peers?
+int check_persist(crl_engine* e) {
+  if (!e->persist_unchecked) return CRL_OK;
+  e->persist_unchecked = false;
+  unsigned gave_up = 0;
+  HIP_TRY(hipMemcpyAsync(&gave_up, e->perr, sizeof gave_up, hipMemcpyDeviceToHost, e->stream));
+  HIP_TRY(hipStreamSynchronize(e->stream));
+  if (gave_up)
+    return fail(CRL_E_DEVICE, "the one-launch shared-table kernel gave up waiting for its workgroups "
+                "(were they all resident?); state and table are not valid - use crl_set_fused_variant(e, 1)");
   return CRL_OK;
 }
 
@@ -890,7 +1007,10 @@ int run_fused(crl_engine* e, int32_t n_steps, bool no_alloc) {
       e->trace_cursor = c > e->trace_cap ? e->trace_cap : (int)c;
     }
   } else {
-    for (int k = 0; k < n_steps; ++k) {
+    bool launched = false;
+    rc = run_persist(e, n_steps, &launched);
+    if (rc) return rc;
+    for (int k = 0; !launched && k < n_steps; ++k) {
       rc = shared_step(e, e->t + (uint64_t)k, e->trace_cursor);
       if (rc) return rc;
       if (e->trace_n > 0 && e->trace_cursor < e->trace_cap) e->trace_cursor += 1;
@@ -968,7 +1088,7 @@ int crl_sync(crl_engine* e) {
   int rc = check_engine(e);
   if (rc) return rc;
   HIP_TRY(hipStreamSynchronize(e->stream));
-  return CRL_OK;
+  return check_persist(e);
 }
 
 int crl_set_maps(crl_engine* e, const uint8_t* cell_class, const int32_t* start,
@@ -1116,7 +1236,7 @@ int crl_get_state(crl_engine* e, int32_t* s, float* reward, uint8_t* done, uint8
   if (ep_step) HIP_TRY(hipMemcpyAsync(ep_step, e->ep_step.p, N * 4, hipMemcpyDeviceToHost, e->stream));
   if (episode) HIP_TRY(hipMemcpyAsync(episode, e->episode.p, N * 4, hipMemcpyDeviceToHost, e->stream));
   HIP_TRY(hipStreamSynchronize(e->stream));
-  return CRL_OK;
+  return check_persist(e);
 }
 
 int crl_set_state(crl_engine* e, const int32_t* s, const int32_t* ep_step, const int32_t* episode) {
@@ -1171,7 +1291,7 @@ int crl_q_get_range(crl_engine* e, int32_t first_table, int32_t count, float* ou
   HIP_TRY(hipMemcpyAsync(out, e->Q.p + (size_t)first_table * e->K, (size_t)count * e->K * sizeof(float),
                          hipMemcpyDeviceToHost, e->stream));
   HIP_TRY(hipStreamSynchronize(e->stream));
-  return CRL_OK;
+  return check_persist(e);
 }
 
 int crl_q_get(crl_engine* e, int32_t table, float* out) { return crl_q_get_range(e, table, 1, out); }
@@ -1224,7 +1344,7 @@ int crl_get_trace(crl_engine* e, int32_t n_steps, int32_t* s_next, uint8_t* acti
   if (reward) HIP_TRY(hipMemcpyAsync(reward, e->trace_r.p, cells * 4, hipMemcpyDeviceToHost, e->stream));
   if (done) HIP_TRY(hipMemcpyAsync(done, e->trace_d.p, cells, hipMemcpyDeviceToHost, e->stream));
   HIP_TRY(hipStreamSynchronize(e->stream));
-  return CRL_OK;
+  return check_persist(e);
 }
 
 int crl_set_exploration_stream(crl_engine* e, int32_t n_steps, const float* u, const int32_t* a_rand) {
@@ -1273,6 +1393,14 @@ int crl_fused_kernel_info(crl_engine* e, int32_t n_steps, char* name, size_t nam
     if (block) *block = p.block;
     if (lds_bytes) *lds_bytes = (int32_t)p.lds;
   } else {
+    const PersistPlan pp = plan_persist(e, n_steps > 0 ? n_steps : 1 << 20);
+    if (pp.ok) {
+      if (name && name_len) snprintf(name, name_len, "k_shared_persist<%d,%d>", e->A, pp.lds_map ? 1 : 2);
+      if (grid) *grid = pp.grid;
+      if (block) *block = 256;
+      if (lds_bytes) *lds_bytes = (int32_t)pp.lds;
+      return CRL_OK;
+    }
     if (name && name_len) snprintf(name, name_len, "k_shared_act+k_reduce_owners");
     if (grid) *grid = (e->N + 255) / 256;
     if (block) *block = 256;
@@ -1297,6 +1425,46 @@ int crl_fused_plan_for_config(const crl_config* cfg, int32_t n_steps, char* name
     return fail(CRL_E_STATE, "launch plan %s: grid %d, block %d, %zu bytes of LDS", p.name, p.grid, p.block, p.lds);
   return CRL_OK;
 }
+
+// Tuning aid: per-phase shader clocks, summed over the steps of the last one-launch
+// shared-table call, of its first (out[0..7]) and last (out[8..15]) workgroup.
+int crl_get_persist_clocks(crl_engine* e, uint64_t* out16) {
+  int rc = check_engine(e);
+  if (rc) return rc;
+  if (!out16) return fail(CRL_E_ARG, "out16 is null");
+  if (!e->perr) return fail(CRL_E_STATE, "no one-launch shared-table kernel has run on this engine");
+  HIP_TRY(hipStreamSynchronize(e->stream));
+  HIP_TRY(hipMemcpy(out16, e->perr + 8, 16 * sizeof(uint64_t), hipMemcpyDeviceToHost));
+  return CRL_OK;
+}
+
+// Measurement helper: nanoseconds per barrier over `n_groups` co-resident workgroups
+// built from device-scope loads and stores (pattern: see k_probe_barrier).
+int crl_probe_barrier(int pattern, int n_groups, int rounds, double* ns_per_barrier) {
+  if (pattern < 0 || pattern > 2 || n_groups < 1 || n_groups > crl::kPersistMaxGroups || rounds < 1 || !ns_per_barrier)
+    return fail(CRL_E_ARG, "pattern 0..2, 1..%d workgroups, rounds >= 1", crl::kPersistMaxGroups);
+  const size_t words = (size_t)(17 + crl::kPersistMaxGroups) * crl::kProbeLine;
+  DevBuf<unsigned> mem;
+  DevBuf<unsigned long long> out;
+  if (mem.alloc(words) != hipSuccess || out.alloc(2) != hipSuccess) return fail(CRL_E_ALLOC, "probe allocation failed");
+  HIP_TRY(hipMemset(mem.p, 0, words * sizeof(unsigned)));
+  HIP_TRY(hipMemset(out.p, 0, 2 * sizeof(unsigned long long)));
+  unsigned* m = mem.p;
+  unsigned long long* o = out.p;
+  void* args[] = {&m, &rounds, &o};
+  const void* kern = pattern == 0   ? reinterpret_cast<const void*>(&crl::k_probe_barrier<0>)
+                     : pattern == 1 ? reinterpret_cast<const void*>(&crl::k_probe_barrier<1>)
+                                    : reinterpret_cast<const void*>(&crl::k_probe_barrier<2>);
+  // co-resident or refused: the workgroups wait for each other
+  HIP_TRY(hipLaunchCooperativeKernel(kern, dim3(n_groups), dim3(256), args, 0, nullptr));
+  HIP_TRY(hipDeviceSynchronize());
+  unsigned long long h[2];
+  HIP_TRY(hipMemcpy(h, out.p, sizeof h, hipMemcpyDeviceToHost));
+  if (h[1]) return fail(CRL_E_DEVICE, "%llu workgroups gave up waiting", h[1]);
+  *ns_per_barrier = (double)h[0] * 10.0 / rounds;  // 100 MHz ticks
+  return CRL_OK;
+}
+
 
 int crl_probe_copy(size_t n_bytes, int repeats) {
   if (n_bytes == 0 || n_bytes % 16 != 0 || repeats < 1) return fail(CRL_E_ARG, "n_bytes must be a positive multiple of 16");

@@ -87,7 +87,7 @@ EXPORTS = [
     "crl_set_state", "crl_get_episode_stats", "crl_get_step_count", "crl_set_step_count", "crl_q_get", "crl_q_set",
     "crl_q_get_range", "crl_set_trace", "crl_get_trace", "crl_set_exploration_stream",
     "crl_device_ptr", "crl_fused_kernel_info", "crl_fused_plan_for_config", "crl_philox4x32_10", "crl_explore_draw",
-    "crl_eps_table", "crl_gen_maps_bernoulli", "crl_gen_maps_noise", "crl_probe_copy",
+    "crl_eps_table", "crl_gen_maps_bernoulli", "crl_gen_maps_noise", "crl_probe_copy", "crl_probe_barrier", "crl_get_persist_clocks",
 ]
 
 
@@ -144,6 +144,8 @@ def load():
     lib.crl_gen_maps_bernoulli.argtypes = [u64, i32, i32, i32, i32, f32, f32, vp, vp]
     lib.crl_gen_maps_noise.argtypes = [u64, i32, i32, i32, i32, f32, f32, f32, vp, vp, vp]
     lib.crl_probe_copy.argtypes = [C.c_size_t, C.c_int]
+    lib.crl_probe_barrier.argtypes = [C.c_int, C.c_int, C.c_int, C.POINTER(C.c_double)]
+    lib.crl_get_persist_clocks.argtypes = [vp, vp]
     _lib = lib
     return lib
 
@@ -192,6 +194,12 @@ def fused_plan_for_config(cfg, n_steps=0):
     g, b, l = C.c_int32(), C.c_int32(), C.c_int32()
     _check(load().crl_fused_plan_for_config(C.byref(cfg), n_steps, name, 128, C.byref(g), C.byref(b), C.byref(l)))
     return dict(name=name.value.decode(), grid=g.value, block=b.value, lds_bytes=l.value)
+
+
+def probe_barrier(pattern, n_groups=256, rounds=2000):
+    ns = C.c_double()
+    _check(load().crl_probe_barrier(pattern, n_groups, rounds, C.byref(ns)))
+    return ns.value
 
 
 def classify_grid(grid, step_reward=-0.01):
@@ -361,6 +369,12 @@ class Engine:
         p = C.c_void_p()
         _check(self.lib.crl_device_ptr(self.h, which, C.byref(p)))
         return p.value
+
+    def persist_clocks(self):
+        """Per-phase shader clocks of the last one-launch shared-table call: (first, last workgroup) x 8."""
+        out = np.zeros(16, np.uint64)
+        _check(self.lib.crl_get_persist_clocks(self.h, _ptr(out)))
+        return out.reshape(2, 8)
 
     def fused_kernel_info(self, n_steps=0):
         """Plan of crl_run_fused(n_steps); 0 = a long launch."""

@@ -130,11 +130,16 @@ int crl_sync(crl_engine* e);
  * launch.  0 = automatic (as many as keep the tables in the last-level cache).
  * Results do not depend on it. */
 int crl_set_resident_envs(crl_engine* e, int32_t n_envs);
-/* Tuning (no reference counterpart): kernel of crl_run_fused for per-env tables.
- * 0 = automatic, 1 = plain (every wave steps envs against tables in HBM),
+/* Tuning (no reference counterpart): kernel of crl_run_fused.  0 = automatic.
+ * Per-env tables: 1 = plain (every wave steps envs against tables in HBM),
  * 2 = hybrid (the last wave of each workgroup steps envs whose whole tables it holds
  * in LDS; used only when 32 tables fit; automatic picks it for launches of at
- * least 64 steps).  Results do not depend on it. */
+ * least 64 steps).  Shared table: 0 and 1 = two launches per step, 2 = all steps of
+ * a call in one launch whose workgroups exchange block sums and table values through
+ * device-scope loads and stores (needs every workgroup resident at once: at most
+ * 65,536 envs and 16,384 table entries, else two launches per step; slower than
+ * those on MI355X, kept for callers that must not launch per step).
+ * Results do not depend on it. */
 int crl_set_fused_variant(crl_engine* e, int32_t variant);
 /* How the last hybrid crl_run_fused split the envs between its two kinds of
  * workers (tables in HBM / tables in LDS); both 0 if the plain kernel ran. */
@@ -272,6 +277,19 @@ int crl_fused_plan_for_config(const crl_config* cfg, int32_t n_steps, char* name
  * kernel `k_probe_copy` moving n_bytes from one device buffer to another, so
  * that hardware traffic counters can be scaled by a launch of known size. */
 int crl_probe_copy(size_t n_bytes, int repeats);
+
+/* Tuning aid (no reference counterpart): per-phase shader clocks, summed over the
+ * steps of the last one-launch shared-table call (crl_set_fused_variant 2), of its
+ * first (out16[0..7]) and last (out16[8..15]) workgroup.  Phases: wait for the
+ * owners' table, act, block sums, drain + publish, wait for the blocks' cells,
+ * cells into the tile, tile sums + publish, loop overhead. */
+int crl_get_persist_clocks(crl_engine* e, uint64_t* out16);
+/* Measurement helper (no reference counterpart): nanoseconds per barrier over
+ * n_groups (<= 256) co-resident workgroups that meet through device-scope loads
+ * and stores.  pattern 0: packed flags, all polled by everybody with 16-byte
+ * loads; 1: one flag per 128-byte line; 2: a tree in which every word has one
+ * writer and one reader. */
+int crl_probe_barrier(int pattern, int n_groups, int rounds, double* ns_per_barrier);
 
 /* -- host-side helpers (no device needed) ----------------------------------- */
 

@@ -31,7 +31,7 @@ def assert_trace_equal(got, want):
                         % (k, bad[0], bad[1], got[k][tuple(bad)], want[k][tuple(bad)]))
 
 
-def run_both(gpu, oracle, cfg, cls, start, n_steps, cr=None, chunks=None, trace_n=None, stream=None):
+def run_both(gpu, oracle, cfg, cls, start, n_steps, cr=None, chunks=None, trace_n=None, stream=None, variant=0):
     N = cfg.n_envs
     trace_n = N if trace_n is None else trace_n
     A, S = cfg.n_actions, cfg.width * cfg.height
@@ -39,6 +39,8 @@ def run_both(gpu, oracle, cfg, cls, start, n_steps, cr=None, chunks=None, trace_
     with gpu.Engine(cfg, 0) as eng:
         eng.set_maps(cls, start, cr)
         eng.set_trace(trace_n, n_steps)
+        if variant:
+            eng.set_fused_variant(variant)
         if stream is not None:
             eng.set_exploration_stream(*stream)
         for c in (chunks or [n_steps]):
@@ -362,16 +364,76 @@ def test_select_step_update_equals_fused(gpu, oracle, shared):
 
 # ---- shared table: ordered reduction ----------------------------------------------
 
+# variant 1: two launches per step; 2: every step of a call in one launch
+@pytest.mark.parametrize("variant", [1, 2])
 @pytest.mark.parametrize("N,W,H,steps,lr", [(64, 4, 4, 50, 0.05), (5000, 16, 16, 120, 0.002),
                                             (5000, 16, 16, 120, 0.05),  # overflows: inf/nan parity
                                             (65536, 64, 64, 12, 0.05)])
-def test_shared_table_matches_oracle(gpu, oracle, N, W, H, steps, lr):
+def test_shared_table_matches_oracle(gpu, oracle, variant, N, W, H, steps, lr):
     cls, start = gpu.gen_maps_bernoulli(2, 1, N, W, H, 0.15)
     cfg = gpu.make_config(N, W, H, table_mode=gpu.TABLE_SHARED, map_mode=gpu.MAP_SHARED, lr=lr,
                           eps0=0.2, episode_len=0, seed=13)
-    _, q = run_both(gpu, oracle, cfg, cls, start, steps, trace_n=min(N, 4096))
+    _, q = run_both(gpu, oracle, cfg, cls, start, steps, trace_n=min(N, 4096), variant=variant)
     if lr < 0.01:
         assert np.isfinite(q).all() and np.count_nonzero(q) > 50
+
+
+def test_shared_table_one_launch_kernel_shapes(gpu, oracle):
+    """The one-launch kernel where its roles do not line up: more owners than blocks
+    of envs (workgroups without envs), a last block that is not full, 8 actions
+    with per-cell rewards and per-env maps read from global memory, calls that
+    alternate (chunked launches)."""
+    # 300 envs = 2 blocks, 1024 keys = 16 owners
+    cls, start = gpu.gen_maps_bernoulli(5, 1, 300, 16, 16, 0.1, 0.03)
+    cfg = gpu.make_config(300, 16, 16, table_mode=gpu.TABLE_SHARED, map_mode=gpu.MAP_SHARED, lr=0.01, eps0=0.3,
+                          episode_len=25, seed=3, trap_reward=-0.5)
+    with gpu.Engine(cfg, 0) as eng:
+        assert eng.fused_kernel_info(10)["name"] == "k_shared_act+k_reduce_owners"
+        eng.set_fused_variant(2)
+        assert eng.fused_kernel_info(10)["name"] == "k_shared_persist<4,1>" and eng.fused_kernel_info(10)["grid"] == 16
+    run_both(gpu, oracle, cfg, cls, start, 90, chunks=[1, 30, 1, 1, 50, 7], variant=2)
+    # 8 actions, cell rewards, per-env maps (global memory), linear epsilon, 1000 envs: last block 232 envs
+    N, W, H = 1000, 24, 20
+    cls, start, cr = gpu.gen_maps_noise(6, N, W, H, 8, 0.2, 0.05, 2.0)
+    cfg = gpu.make_config(N, W, H, n_actions=8, table_mode=gpu.TABLE_SHARED, lr=0.004, eps_mode=gpu.EPS_EPISODE_LINEAR,
+                          eps0=0.9, eps_end=0.1, eps_span=4, episode_len=40, seed=8,
+                          reward_flags=gpu.REWARD_CELLS | gpu.REWARD_BASE_CELLS)
+    with gpu.Engine(cfg, 0) as eng:
+        eng.set_fused_variant(2)
+        assert eng.fused_kernel_info(10)["name"] == "k_shared_persist<8,2>"
+    tr, q = run_both(gpu, oracle, cfg, cls, start, 130, cr=cr, chunks=[64, 66], variant=2)
+    assert len(np.unique(tr["action"])) == 8 and np.isfinite(q).all()
+    # goal test on the resulting cell, sticky done, zero-floored max, supplied stream
+    N, W, H = 700, 9, 7
+    cls, start = gpu.gen_maps_bernoulli(7, 1, N, W, H, 0.1)
+    cfg = gpu.make_config(N, W, H, table_mode=gpu.TABLE_SHARED, map_mode=gpu.MAP_SHARED, lr=0.01, eps0=0.25,
+                          auto_reset=0, goal_mode=gpu.GOAL_ON_RESULT, max_mode=gpu.MAX_ZERO_FLOOR, seed=5)
+    rng = np.random.default_rng(1)
+    u = rng.random((45, N), dtype=np.float32)  # (the oracle takes a stream that covers the whole run)
+    a = rng.integers(0, 4, (45, N)).astype(np.int32)
+    run_both(gpu, oracle, cfg, cls, start, 45, stream=(u, a), chunks=[20, 25], variant=2)
+    # episode budget and return accumulators
+    N, W, H, T, E = 600, 8, 8, 200, 3
+    cls, start = gpu.gen_maps_bernoulli(15, 1, N, W, H, 0.1, 0.04)
+    cfg = gpu.make_config(N, W, H, episode_len=19, eps0=0.35, seed=12, lr=0.002, table_mode=gpu.TABLE_SHARED,
+                          map_mode=gpu.MAP_SHARED, max_episodes=E, track_returns=1)
+    Q = np.zeros((1, W * H, 4), np.float32)
+    ost, ostats = oracle.new_state(cfg, start), oracle.new_stats(N)
+    want = oracle.run(cfg, cls, None, start, Q, ost, 0, T, trace_n=N, stats=ostats)
+    with gpu.Engine(cfg, 0) as eng:
+        eng.set_maps(cls, start)
+        eng.set_trace(N, T)
+        eng.set_fused_variant(2)
+        eng.run_fused(120)
+        eng.run_fused(T - 120)
+        assert_trace_equal(eng.get_trace(T), want)
+        st, stats = eng.get_state(), eng.episode_stats()
+        assert_q_close(eng.q_get(0, 1).reshape(Q.shape), Q)
+    for k in ("s", "ep_step", "episode", "reward", "done", "action"):
+        assert np.array_equal(st[k], ost[k]), k
+    for k in ("last_return", "last_length", "return_sum", "length_sum"):
+        assert np.array_equal(stats[k], ostats[k]), k
+    assert (ost["episode"] == E).all()
 
 
 def test_shared_table_all_envs_on_one_cell(gpu, oracle):

@@ -18,12 +18,14 @@ def free_device_bytes():
     return free.value
 
 
-def run_pair(gpu, cfg, cls, start, chunks, n_tables):
+def run_pair(gpu, cfg, cls, start, chunks, n_tables, variant=0):
     """-> (state, tables) after the launches in `chunks`, once per entry point"""
     out = []
     for noalloc in (False, True):
         with gpu.Engine(cfg, 0) as eng:
             eng.set_maps(cls, start)
+            if variant:
+                eng.set_fused_variant(variant)
             eng.sync()
             before = free_device_bytes()
             for c in chunks:
@@ -57,8 +59,9 @@ def test_noalloc_shared_table_two_calls_second_smaller(gpu):
         cls, start = gpu.gen_maps_bernoulli(2, 1, N, W, H, 0.15)
         cfg = gpu.make_config(N, W, H, table_mode=gpu.TABLE_SHARED, map_mode=gpu.MAP_SHARED, lr=0.002,
                               eps0=0.2, episode_len=50, seed=13)
-        st, q = run_pair(gpu, cfg, cls, start, (steps,), 1)
-        assert np.isfinite(q).all() and np.count_nonzero(q) > 100
+        for variant in (0, 2):  # two launches per step; all steps in one launch (its flags, too, come from the scratch)
+            st, q = run_pair(gpu, cfg, cls, start, (steps,), 1, variant)
+            assert np.isfinite(q).all() and np.count_nonzero(q) > 100
 
 
 def test_noalloc_rejects_a_reduction_larger_than_the_scratch(gpu):
