@@ -203,8 +203,9 @@ int crl_run_fused(crl_engine* e, int32_t n_steps);
  * under HIP graph capture, tight serving loops, harnesses that forbid
  * hipMalloc): no counterpart in the reference.  Same results as crl_run_fused,
  * but its scratch - the ticket counters of the per-env kernels, the hand-off
- * cells of the shared table's ordered reduction - lives in a static device
- * array of 8 MB + 256 bytes that each GPU the library runs on holds until the
+ * cells of the shared table's ordered reduction, the step flags of the one-launch
+ * shared-table kernel - lives in a static device
+ * array of 8 MB + 4 KB that each GPU the library runs on holds until the
  * process ends, and the call allocates and frees nothing (device or host).
  * CRL_E_RANGE if the engine's reduction needs more hand-off cells than the
  * array holds (65,536 envs on a 64x64x4 table need 4 MB).  All engines on one
