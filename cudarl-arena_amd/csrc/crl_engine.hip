@@ -279,6 +279,7 @@ struct FusedPlan {
   bool moves;      // ... whose table waves read pre-built move codes from LDS
   bool fixed;      // every pair of tickets has its own wave: dealt by position, no counter
   bool pair;       // per-env kernel: two lanes per env
+  int pair_envs;   // ticket kernel: envs per thin table wave (32, 16, 8), 0: 64-env waves
   bool rich;       // ticket kernel: the folded loop's variant with per-cell rewards / per-episode epsilon
   int tab_stride;  // floats between two tables in LDS
 };
@@ -405,11 +406,18 @@ FusedPlan plan_fused(const crl_engine* e, int n_steps) {
       // Few enough envs that 32-env waves still find a SIMD each: one ticket per wave,
       // two lanes per env - half the distinct addresses per request and the Philox
       // rounds shared by the pair (32x32 maps: 4096 envs +10 %, 8192 +8 %, 16,384 +0 %)
+      long units = tickets;  // tickets as the kernel counts them
       if (p.moves && waves == 1 && tickets <= 2 * kComputeUnits) {
         p.pair = true;
-        p.grid = (int)std::min<long>(std::max<long>(1, resident / 32), tickets);
+        // ... and thinner still while that gives more compute units a wave of their own
+        // (4096 envs of 32x32: 128 waves of 32 envs 1.165e10 env-steps/s, 256 of 16 1.25e10,
+        // 512 of 8 - two to a unit - 1.16e10)
+        p.pair_envs = crl::kTicketEnvs;
+        while (p.pair_envs > 8 && (e->N + p.pair_envs - 1) / p.pair_envs < kComputeUnits) p.pair_envs /= 2;
+        units = (e->N + p.pair_envs - 1) / p.pair_envs;
+        p.grid = (int)std::min<long>(std::max<long>(1, resident / p.pair_envs), units);
       }
-      p.fixed = (long)p.grid * waves * (p.pair ? 1 : 2) >= tickets && n_steps < kHybridMinSteps;  // a wave for every pair of tickets
+      p.fixed = (long)p.grid * waves * (p.pair ? 1 : 2) >= units && n_steps < kHybridMinSteps;  // a wave for every pair of tickets
       p.lds = waves * (p.moves ? mv_lds : map_lds);
     }
   }
@@ -445,7 +453,7 @@ void launch_fused_a(const crl_engine* e, const FusedPlan& p, uint64_t t0, int n)
     unsigned* tk = e->tk;
 #define CRL_LAUNCH_TICKETS(MODE, LDSW, MOVES)                                                       \
   hipLaunchKernelGGL((crl::k_fused_tickets<A, MODE, LDSW, MOVES>), g, b, p.lds, e->stream, R, P, t0, n, \
-                     tk, p.tab_stride, p.fixed ? 1 : 0, p.pair ? 1 : 0)
+                     tk, p.tab_stride, p.fixed ? 1 : 0, p.pair ? p.pair_envs : 0)
     if (p.rich && p.moves)
       CRL_LAUNCH_TICKETS(2, false, true);
     else if (p.rich)

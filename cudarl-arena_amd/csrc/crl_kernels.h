@@ -571,7 +571,7 @@ __global__ __launch_bounds__(LDSW ? 320 : 256) void k_fused_tickets(const Rules 
                                                                      unsigned* __restrict__ ticket,
                                                                      const int tab_stride,
                                                                      const int fixed_tickets,
-                                                                     const int pair_tables) {
+                                                                     const int pair_envs) {
   constexpr bool FAST = MODE >= 1;  // the folded loop ...
   constexpr bool RICH = MODE == 2;  // ... in its variant with per-cell rewards and per-episode epsilon
   extern __shared__ uint32_t lds[];
@@ -585,10 +585,12 @@ __global__ __launch_bounds__(LDSW ? 320 : 256) void k_fused_tickets(const Rules 
   const int lds_slice = !LDSW ? 0 : FAST ? P.mv_words * kTicketEnvs : P.map_words * 64;
   uint32_t* my_words = lds + wave * slice;  // (the LDS wave is the last one)
   float* tabs = reinterpret_cast<float*>(lds + (n_waves - 1) * slice + lds_slice);
-  const unsigned n_tickets = (unsigned)((P.N + kTicketEnvs - 1) / kTicketEnvs);
-  // (pair_tables: the table waves, too, take one ticket and give every env two lanes)
-  const bool thin = lds_worker || (FAST && MOVES && pair_tables);
-  const int cap = thin ? kTicketEnvs : 64;
+  // envs per ticket: 32, or what a thin table wave steps (never with an LDS wave beside it)
+  const int unit = (FAST && MOVES && pair_envs) ? pair_envs : kTicketEnvs;
+  const unsigned n_tickets = (unsigned)((P.N + unit - 1) / unit);
+  // (pair_envs: the table waves, too, take one ticket and give every env several lanes)
+  const bool thin = lds_worker || (FAST && MOVES && pair_envs);
+  const int cap = thin ? unit : 64;
   const unsigned take = thin ? 1u : 2u;
   const size_t table = P.S * A;  // floats per table
 
@@ -608,7 +610,7 @@ __global__ __launch_bounds__(LDSW ? 320 : 256) void k_fused_tickets(const Rules 
       base = __shfl(base, 0);
     }
     if (base >= n_tickets) break;  // every worker gets here: the counter only grows
-    const int env0 = (int)base * kTicketEnvs;
+    const int env0 = (int)base * unit;
     const int n_here = min(cap, P.N - env0);
     const int env = env0 + lane;
     const bool live = lane < n_here;
@@ -626,12 +628,13 @@ __global__ __launch_bounds__(LDSW ? 320 : 256) void k_fused_tickets(const Rules 
     if (!lds_worker) {
       __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
       __builtin_amdgcn_wave_barrier();
-      if (kTableMoves && pair_tables) {
-        const int l = lane & (kTicketEnvs - 1);
+      if (kTableMoves && pair_envs) {
+        // lanes l, l + unit, ... step env l; the halves of the wave share the Philox rounds
+        const int l = lane & (unit - 1);
         if (l < n_here) {
           const GlobalTable<A> tab{P.Q + (size_t)(env0 + l) * table};
           if (n_steps >= kTouchMinSteps) tab.touch((int)table);
-          run_env_fast<A, true, RICH>(R, P, env0 + l, t0, n_steps, MovesLds<A>{my_words + l, kTicketEnvs},
+          run_env_fast<A, true, RICH>(R, P, env0 + l, t0, n_steps, MovesLds<A>{my_words + l, unit},
                                       RICH && P.cell_reward ? P.cell_reward + (size_t)(env0 + l) * P.S : nullptr,
                                       tab);
         }

@@ -196,8 +196,8 @@ def test_every_valid_configuration_has_a_launch_plan_that_fits(pycrl):
     assert pycrl.fused_plan_for_config(c4, 1000) == dict(name="k_fused_tickets<4,fast,hbm+lds>", grid=256, block=256,
                                                          lds_bytes=152064)
     c2 = pycrl.make_config(4096, 32, 32, episode_len=256)
-    assert pycrl.fused_plan_for_config(c2, 10000) == dict(name="k_fused_tickets<4,fast,hbm>", grid=128, block=64,
-                                                          lds_bytes=65536)
+    assert pycrl.fused_plan_for_config(c2, 10000) == dict(name="k_fused_tickets<4,fast,hbm>", grid=256, block=64,
+                                                          lds_bytes=65536)  # 16 envs to a wave: a wave per compute unit
     with pytest.raises(pycrl.CrlError):
         pycrl.fused_plan_for_config(pycrl.make_config(64, 8, 8, table_mode=pycrl.TABLE_SHARED), 10)
 
