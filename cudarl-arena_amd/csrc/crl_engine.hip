@@ -142,6 +142,7 @@ struct crl_engine {
   unsigned* perr = nullptr;
   bool persist_unchecked = false;
   bool persist_refused = false;  // the device refused the co-resident launch once: not tried again
+  int persist_spin_limit = crl::kPersistSpinLimit;  // polls a workgroup waits for its peers before it gives up
 
   DevBuf<int32_t> s, ep_step, episode, start, act;
   DevBuf<float> reward;
@@ -672,7 +673,8 @@ hipError_t launch_persist_kernel(crl_engine* e, const PersistPlan& p, int n_step
   crl::ReduceGeom G = p.G;
   uint2* handoff = e->ho;
   unsigned* err = e->perr;
-  void* args[] = {&R, &P, &t0, &n, &trace_row0, &key, &delta, &G, &handoff, &flags, &err};
+  int spin_limit = e->persist_spin_limit;
+  void* args[] = {&R, &P, &t0, &n, &trace_row0, &key, &delta, &G, &handoff, &flags, &err, &spin_limit};
   // a cooperative launch is refused unless all workgroups can be resident together,
   // which the kernel's waits rely on
   return hipLaunchCooperativeKernel(reinterpret_cast<const void*>(&crl::k_shared_persist<A, MAP>), dim3(p.grid),
@@ -1353,6 +1355,13 @@ int crl_get_trace(crl_engine* e, int32_t n_steps, int32_t* s_next, uint8_t* acti
   if (done) HIP_TRY(hipMemcpyAsync(done, e->trace_d.p, cells, hipMemcpyDeviceToHost, e->stream));
   HIP_TRY(hipStreamSynchronize(e->stream));
   return check_persist(e);
+}
+
+int crl_set_persist_spin_limit(crl_engine* e, int32_t polls) {
+  if (!e) return fail(CRL_E_ARG, "null engine");
+  if (polls < 1) return fail(CRL_E_ARG, "at least one poll");
+  e->persist_spin_limit = polls;
+  return CRL_OK;
 }
 
 int crl_set_exploration_stream(crl_engine* e, int32_t n_steps, const float* u, const int32_t* a_rand) {

@@ -25,8 +25,8 @@
 // owner has consumed the cells of step k, and an owner overwrites its table values
 // only after step 4's wait, when every block has read them: one buffer of each.
 //
-// Every wait is bounded: a workgroup that waits for kPersistSpinLimit polls sets
-// the error word and leaves; the others then leave, too.
+// Every wait is bounded: a workgroup that waits for `spin_limit` polls (default
+// kPersistSpinLimit) sets the error word and leaves; the others then leave, too.
 #pragma once
 #include "crl_kernels.h"
 
@@ -137,7 +137,7 @@ __device__ __forceinline__ void load_rows_dev<8>(const float* Q, int cell, const
 // Wave 0 polls the first `n` flags until all have reached `want` (or the limit is
 // hit, or another workgroup has given up); every thread returns the same answer.
 __device__ __forceinline__ bool wait_flags(const unsigned* flags, int n, unsigned want, unsigned* err,
-                                           int* lds_dead) {
+                                           int* lds_dead, const int spin_limit) {
   if (threadIdx.x < 64) {
     const int i0 = (int)threadIdx.x * 4;
     bool ok = true;
@@ -148,7 +148,7 @@ __device__ __forceinline__ bool wait_flags(const unsigned* flags, int n, unsigne
         ok = (int)(v.x - want) >= 0 && (i0 + 1 >= n || (int)(v.y - want) >= 0) &&
              (i0 + 2 >= n || (int)(v.z - want) >= 0) && (i0 + 3 >= n || (int)(v.w - want) >= 0);
         if (ok) break;
-        if (++spins >= kPersistSpinLimit || ((spins & 255) == 0 && ld_dev(err) != 0u)) break;
+        if (++spins >= spin_limit || ((spins & 255) == 0 && ld_dev(err) != 0u)) break;
       }
     }
     if (!__all(ok) && threadIdx.x == 0) {
@@ -246,7 +246,8 @@ template <int A, int MAP>
 __global__ __launch_bounds__(256) void k_shared_persist(const Rules R, const Ptrs P, const uint64_t t0,
                                                          const int n_steps, const int trace_row0,
                                                          int32_t* key, float* delta, const ReduceGeom G,
-                                                         uint2* handoff, unsigned* flags, unsigned* err) {
+                                                         uint2* handoff, unsigned* flags, unsigned* err,
+                                                         const int spin_limit) {
   extern __shared__ unsigned char lds_raw[];
   ReduceLds& L = *reinterpret_cast<ReduceLds*>(lds_raw);
   float* tile = reinterpret_cast<float*>(lds_raw);  // the owner's [block][key] tile reuses the block's table
@@ -292,7 +293,7 @@ __global__ __launch_bounds__(256) void k_shared_persist(const Rules R, const Ptr
     const uint64_t t = t0 + (uint64_t)k;
     CRL_MARK(7);
     // 1. the table of this step: every owner has published its values of step k
-    if (k > 0 && !wait_flags(owner_flags, n_own, (unsigned)k, err, &lds_dead)) break;
+    if (k > 0 && !wait_flags(owner_flags, n_own, (unsigned)k, err, &lds_dead, spin_limit)) break;
     CRL_MARK(0);
     reduce_block_clear(L, G);
 
@@ -375,7 +376,7 @@ __global__ __launch_bounds__(256) void k_shared_persist(const Rules R, const Ptr
 
     // 4. as owner of 64 keys: all blocks' cells, added in tree order
     if (is_owner) {
-      if (!wait_flags(block_flags, n_groups, (unsigned)(k + 1), err, &lds_dead)) break;
+      if (!wait_flags(block_flags, n_groups, (unsigned)(k + 1), err, &lds_dead, spin_limit)) break;
       CRL_MARK(4);
       // (the wait's barrier also ends every thread's use of the block's LDS table)
       const int b = tid;

@@ -85,7 +85,7 @@ EXPORTS = [
     "crl_set_stream", "crl_sync", "crl_set_resident_envs", "crl_set_fused_variant", "crl_get_fused_split", "crl_set_maps", "crl_set_cell", "crl_classify_grid", "crl_reset",
     "crl_step", "crl_select", "crl_update", "crl_td_update", "crl_run_fused", "crl_run_fused_noalloc", "crl_get_state",
     "crl_set_state", "crl_get_episode_stats", "crl_get_step_count", "crl_set_step_count", "crl_q_get", "crl_q_set",
-    "crl_q_get_range", "crl_set_trace", "crl_get_trace", "crl_set_exploration_stream",
+    "crl_q_get_range", "crl_set_trace", "crl_get_trace", "crl_set_exploration_stream", "crl_set_persist_spin_limit",
     "crl_device_ptr", "crl_fused_kernel_info", "crl_fused_plan_for_config", "crl_philox4x32_10", "crl_explore_draw",
     "crl_eps_table", "crl_gen_maps_bernoulli", "crl_gen_maps_noise", "crl_probe_copy", "crl_probe_barrier", "crl_get_persist_clocks",
 ]
@@ -131,6 +131,7 @@ def load():
     lib.crl_set_trace.argtypes = [vp, i32, i32]
     lib.crl_get_trace.argtypes = [vp, i32, vp, vp, vp, vp]
     lib.crl_set_exploration_stream.argtypes = [vp, i32, vp, vp]
+    lib.crl_set_persist_spin_limit.argtypes = [vp, i32]
     lib.crl_device_ptr.argtypes = [vp, i32, C.POINTER(vp)]
     lib.crl_fused_kernel_info.argtypes = [vp, i32, C.c_char_p, C.c_size_t, C.POINTER(i32), C.POINTER(i32),
                                           C.POINTER(i32)]
@@ -369,6 +370,9 @@ class Engine:
         p = C.c_void_p()
         _check(self.lib.crl_device_ptr(self.h, which, C.byref(p)))
         return p.value
+
+    def set_persist_spin_limit(self, polls):
+        _check(self.lib.crl_set_persist_spin_limit(self.h, polls))
 
     def persist_clocks(self):
         """Per-phase shader clocks of the last one-launch shared-table call: (first, last workgroup) x 8."""

@@ -253,6 +253,15 @@ int crl_get_trace(crl_engine* e, int32_t n_steps, int32_t* s_next, uint8_t* acti
 int crl_set_exploration_stream(crl_engine* e, int32_t n_steps, const float* u,
                                const int32_t* a_rand);
 
+/* How many polls a workgroup of the one-launch shared-table kernel waits for its
+ * peers before it gives up (default 2^20, a few hundred milliseconds).  A workgroup
+ * that gives up sets a word that the others see and leave on; the next call that
+ * synchronises (crl_sync, crl_get_state, crl_q_get, crl_get_trace) then fails with
+ * CRL_E_DEVICE and the engine's state and table are not valid any more.  With a
+ * limit of 1 every workgroup leaves at its first unanswered poll: how the tests
+ * exercise that path without a kernel that hangs. */
+int crl_set_persist_spin_limit(crl_engine* e, int32_t polls);
+
 /* raw device pointers of the SoA state for zero-copy consumers; index with
  * CRL_PTR_*.  Valid until crl_destroy. */
 enum {

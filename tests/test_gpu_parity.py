@@ -436,6 +436,34 @@ def test_shared_table_one_launch_kernel_shapes(gpu, oracle):
     assert (ost["episode"] == E).all()
 
 
+def test_shared_table_one_launch_kernel_gives_up_cleanly(gpu):
+    """Failure handling of the one-launch kernel, forced from the host: with a wait of
+    one poll the workgroups do not find their peers' flags, give up, and every one of
+    them leaves the kernel; the next synchronising call reports it, and the device is
+    fine afterwards."""
+    N, W, H = 20000, 32, 32
+    cls, start = gpu.gen_maps_bernoulli(6, 1, N, W, H, 0.15)
+    cfg = gpu.make_config(N, W, H, table_mode=gpu.TABLE_SHARED, map_mode=gpu.MAP_SHARED, lr=0.004, eps0=0.2, seed=21)
+    with gpu.Engine(cfg, 0) as eng:
+        eng.set_maps(cls, start)
+        eng.set_fused_variant(2)
+        eng.set_persist_spin_limit(1)
+        eng.run_fused(50)  # asynchronous: the launch itself succeeds
+        with pytest.raises(gpu.CrlError) as err:
+            eng.sync()
+        assert err.value.code == -2 and "gave up" in str(err.value)
+        eng.sync()  # reported once
+    with gpu.Engine(cfg, 0) as eng:  # same device, default limit: all is well
+        eng.set_maps(cls, start)
+        eng.set_fused_variant(2)
+        eng.run_fused(50)
+        q_one = eng.q_get(0)
+    with gpu.Engine(cfg, 0) as eng:
+        eng.set_maps(cls, start)
+        eng.run_fused(50)
+        assert np.array_equal(eng.q_get(0), q_one) and np.isfinite(q_one).all()
+
+
 def test_shared_table_all_envs_on_one_cell(gpu, oracle):
     """Degenerate segment: every env hits the same (s,a) keys."""
     N, W, H = 3000, 3, 3
