@@ -22,16 +22,13 @@
 
 namespace {
 
-thread_local std::string g_err;
-
 int fail(int code, const char* fmt, ...) {
   char buf[512];
   va_list ap;
   va_start(ap, fmt);
   vsnprintf(buf, sizeof buf, fmt, ap);
   va_end(ap);
-  g_err = buf;
-  return code;
+  return crl::fail_with(code, buf);
 }
 
 #define HIP_TRY(expr)                                                                   \
@@ -795,7 +792,7 @@ int opt_in_ticket_kernels(crl_engine* e);
 int create_engine(const crl_config* cfg, int device, crl_engine** out) {
   if (!out) return fail(CRL_E_ARG, "out is null");
   *out = nullptr;
-  int rc = crl::validate_config(cfg, g_err);
+  int rc = crl::validate_config(cfg, crl::last_error());
   if (rc != CRL_OK) return rc;
   int ndev = 0;
   hipError_t herr = hipGetDeviceCount(&ndev);
@@ -1037,7 +1034,7 @@ int run_fused(crl_engine* e, int32_t n_steps, bool no_alloc) {
 
 extern "C" {
 
-const char* crl_last_error(void) { return g_err.c_str(); }
+const char* crl_last_error(void) { return crl::last_error().c_str(); }
 const char* crl_version(void) { return CRL_VERSION; }
 
 int crl_device_count(void) {
@@ -1428,7 +1425,7 @@ int crl_fused_kernel_info(crl_engine* e, int32_t n_steps, char* name, size_t nam
 
 int crl_fused_plan_for_config(const crl_config* cfg, int32_t n_steps, char* name, size_t name_len,
                               int32_t* grid, int32_t* block, int32_t* lds_bytes) {
-  int rc = crl::validate_config(cfg, g_err);
+  int rc = crl::validate_config(cfg, crl::last_error());
   if (rc != CRL_OK) return rc;
   if (cfg->table_mode != CRL_TABLE_PER_ENV) return fail(CRL_E_ARG, "only per-env tables have a fused launch plan");
   crl_engine shell;  // sizes only: nothing is allocated and no device is touched

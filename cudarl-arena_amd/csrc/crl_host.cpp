@@ -13,6 +13,20 @@
 
 namespace crl {
 
+std::string& last_error() {
+  thread_local std::string text;
+  return text;
+}
+
+int fail_with(int code, const char* why) {
+  try {
+    last_error() = why;
+  } catch (...) {  // out of memory for the text: the code still says what happened
+  }
+  return code;
+}
+
+
 int validate_config(const crl_config* c, std::string& why) {
   char buf[256];
   auto bad = [&](int code, const char* msg) {
@@ -163,22 +177,22 @@ void crl_explore_draw(uint64_t seed, uint32_t env, uint64_t t, int32_t n_actions
 }
 
 int crl_eps_table(const crl_config* cfg, float* out, int32_t cap, int32_t* len) {
-  std::string why;
-  if (crl::validate_config(cfg, why) != CRL_OK) return CRL_E_ARG;
+  const int rc = crl::validate_config(cfg, crl::last_error());
+  if (rc != CRL_OK) return rc;
   try {
     const std::vector<float> tab = crl::build_eps_table(*cfg);
     if (len) *len = (int32_t)tab.size();
     if (out)
       for (int32_t i = 0; i < cap && (size_t)i < tab.size(); ++i) out[i] = tab[(size_t)i];
   } catch (...) {
-    return CRL_E_ALLOC;
+    return crl::fail_with(CRL_E_ALLOC, "crl_eps_table: host allocation failed");
   }
   return CRL_OK;
 }
 
 int crl_classify_grid(const float* grid, size_t n, float step_reward, uint8_t* out_class,
                       float* out_reward) {
-  if (!grid || !out_class) return CRL_E_ARG;
+  if (!grid || !out_class) return crl::fail_with(CRL_E_ARG, "crl_classify_grid: null array");
   for (size_t i = 0; i < n; ++i) {
     const float v = grid[i];
     uint8_t k;
@@ -203,10 +217,13 @@ int crl_classify_grid(const float* grid, size_t n, float step_reward, uint8_t* o
 int crl_gen_maps_bernoulli(uint64_t seed, int32_t n_maps, int32_t n_envs, int32_t width,
                            int32_t height, float p_wall, float p_trap, uint8_t* cell_class,
                            int32_t* start) {
-  if (n_maps < 1 || n_envs < 1 || width < 1 || height < 1 || !cell_class || !start) return CRL_E_ARG;
-  if (n_maps != 1 && n_maps != n_envs) return CRL_E_ARG;
+  if (n_maps < 1 || n_envs < 1 || width < 1 || height < 1 || !cell_class || !start)
+    return crl::fail_with(CRL_E_ARG, "crl_gen_maps_bernoulli: sizes must be >= 1 and the arrays not null");
+  if (n_maps != 1 && n_maps != n_envs)
+    return crl::fail_with(CRL_E_ARG, "crl_gen_maps_bernoulli: one shared map or one map per env");
+  if ((int64_t)width * height < 2 || (int64_t)width * height > ((int64_t)1 << 30))
+    return crl::fail_with(CRL_E_ARG, "crl_gen_maps_bernoulli: a map has 2 to 2^30 cells");
   const int S = width * height;
-  if (S < 2) return CRL_E_ARG;
   try {
   std::vector<int> n_free((size_t)n_maps), goal((size_t)n_maps);
   bool ok = crl::parallel_for(n_maps, [&](int m) {
@@ -248,19 +265,23 @@ int crl_gen_maps_bernoulli(uint64_t seed, int32_t n_maps, int32_t n_envs, int32_
       start[i] = free_cells[crl::below(sg.word(4), nf)];
     }) && ok;
   }
-  return ok ? CRL_OK : CRL_E_ALLOC;
+  return ok ? CRL_OK : crl::fail_with(CRL_E_ALLOC, "crl_gen_maps_bernoulli: host allocation or a worker thread failed");
   } catch (...) {
-    return CRL_E_ALLOC;
+    return crl::fail_with(CRL_E_ALLOC, "crl_gen_maps_bernoulli: host allocation failed");
   }
 }
 
 int crl_gen_maps_noise(uint64_t seed, int32_t n_maps, int32_t width, int32_t height, int32_t pitch,
                        float wall_frac, float sigma, float goal_bonus, uint8_t* cell_class,
                        int32_t* start, float* cell_reward) {
-  if (n_maps < 1 || width < 1 || height < 1 || pitch < 1 || !cell_class || !start) return CRL_E_ARG;
-  if (!(wall_frac >= 0.0f && wall_frac < 1.0f)) return CRL_E_ARG;
+  if (n_maps < 1 || width < 1 || height < 1 || pitch < 1 || !cell_class || !start)
+    return crl::fail_with(CRL_E_ARG, "crl_gen_maps_noise: sizes must be >= 1 and the arrays not null");
+  if (!(wall_frac >= 0.0f && wall_frac < 1.0f))
+    return crl::fail_with(CRL_E_ARG, "crl_gen_maps_noise: wall_frac must be in [0, 1)");
+  if ((int64_t)width * height > ((int64_t)1 << 30))
+    return crl::fail_with(CRL_E_ARG, "crl_gen_maps_noise: a map has at most 2^30 cells");
   const int S = width * height;
-  if (S < 2) return CRL_E_ARG;
+  if (S < 2) return crl::fail_with(CRL_E_ARG, "crl_gen_maps_noise: a map needs two cells");
   const int lw = (width + pitch - 1) / pitch + 1, lh = (height + pitch - 1) / pitch + 1;
   const bool ok = crl::parallel_for(n_maps, [&](int m) {
     uint8_t* cls = cell_class + (size_t)m * S;
@@ -309,7 +330,7 @@ int crl_gen_maps_noise(uint64_t seed, int32_t n_maps, int32_t width, int32_t hei
       cr[g] += goal_bonus;
     }
   });
-  return ok ? CRL_OK : CRL_E_ALLOC;
+  return ok ? CRL_OK : crl::fail_with(CRL_E_ALLOC, "crl_gen_maps_noise: host allocation or a worker thread failed");
 }
 
 }  // extern "C"

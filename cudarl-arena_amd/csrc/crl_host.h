@@ -10,6 +10,11 @@
 
 namespace crl {
 
+// The calling thread's last failure text, behind crl_last_error().
+std::string& last_error();
+// Notes `why` as the thread's last failure and returns `code`.
+int fail_with(int code, const char* why);
+
 // CRL_OK, or a negative status with the reason in `why`
 int validate_config(const crl_config* cfg, std::string& why);
 

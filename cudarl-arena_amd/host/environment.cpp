@@ -56,11 +56,11 @@ Environment::Environment(int id, int width, int height) : env_id(id), engine(nul
   cfg.eps0 = 0.0f;
   cfg.eps_span = 1;
   cfg.seed = (uint64_t)id;
-  check(crl_create(&cfg, 0, &engine), "Environment: crl_create");
-
+  // (host buffers first: nothing below may throw while the engine is held by a raw pointer)
   std::vector<uint8_t> cls(grid_store.size());
   std::vector<float> rew(grid_store.size());
   crl_classify_grid(grid_store.data(), grid_store.size(), -0.01f, cls.data(), rew.data());
+  check(crl_create(&cfg, 0, &engine), "Environment: crl_create");
   const int32_t start = (height / 2) * width + width / 2;  // src/environment.cu:9-10
   int rc = crl_set_maps(engine, cls.data(), &start, rew.data());
   if (rc != CRL_OK) {

@@ -94,8 +94,26 @@ Array load(const std::string& path) {
     if (c == ',') c = ' ';
   std::istringstream ds(dims);
   int64_t d;
-  while (ds >> d) a.shape.push_back(d);
-  const size_t n = count(a.shape);
+  while (ds >> d) {
+    if (d < 0) throw std::runtime_error(path + ": negative dimension in header");
+    a.shape.push_back(d);
+  }
+  // the header's word is checked against the file before anything is allocated
+  const std::streamoff at = f.tellg();
+  f.seekg(0, std::ios::end);
+  const std::streamoff left = f.tellg() - at;
+  f.seekg(at);
+  const size_t elem = a.is_double ? sizeof(double) : sizeof(float);
+  const size_t max_elems = left > 0 ? (size_t)left / elem : 0;
+  size_t n = 1;
+  for (int64_t dim : a.shape) {
+    if (dim == 0) {
+      n = 0;
+      break;
+    }
+    if (n > max_elems / (size_t)dim) throw std::runtime_error(path + ": truncated data");
+    n *= (size_t)dim;
+  }
   if (a.is_double) {
     a.f64.resize(n);
     f.read(reinterpret_cast<char*>(a.f64.data()), (std::streamsize)(n * sizeof(double)));

@@ -31,9 +31,11 @@ CudaQLearning::CudaQLearning(int width, int height, int action_space_size, float
   cfg.trap_reward = -1.0f;
   cfg.eps_mode = CRL_EPS_FIXED;
   cfg.eps_span = 1;
+  if (width < 1 || height < 1 || action_space_size < 1)
+    throw std::runtime_error("CudaQLearning: width, height and action_space_size must be >= 1");
+  h_q_table.resize((size_t)width * height * action_space_size, 0.0f);  // (before the engine: may throw)
   if (crl_create(&cfg, 0, &engine) != CRL_OK)  // src/q_learning.cu:17-19
     throw std::runtime_error(std::string("Failed to allocate device memory for Q-table: ") + crl_last_error());
-  h_q_table.resize((size_t)width * height * action_space_size, 0.0f);
   if (std::getenv("CUDARL_VERBOSE"))
     std::cout << "CudaQLearning initialized with " << width << "x" << height << " states and "
               << action_space_size << " actions" << std::endl;

@@ -5,6 +5,7 @@
 #include <cstdio>
 #include <ostream>
 #include <stdexcept>
+#include <string>
 
 namespace cudarl {
 
@@ -77,9 +78,11 @@ TrainMetrics train(BatchedEnvironment& env, int num_episodes, int max_steps, std
   std::vector<float> eps_tab;
   {
     int32_t len = 0;
-    crl_eps_table(&env.config(), nullptr, 0, &len);
+    if (crl_eps_table(&env.config(), nullptr, 0, &len) != CRL_OK || len < 1)
+      throw std::runtime_error(std::string("train: epsilon table: ") + crl_last_error());
     eps_tab.resize((size_t)len);
-    crl_eps_table(&env.config(), eps_tab.data(), len, &len);
+    if (crl_eps_table(&env.config(), eps_tab.data(), len, &len) != CRL_OK)
+      throw std::runtime_error(std::string("train: epsilon table: ") + crl_last_error());
   }
   const int log_every = std::max(1, num_episodes / 20);  // src/train.py:236
   int next_log = log_every;

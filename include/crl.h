@@ -190,7 +190,10 @@ int crl_update(crl_engine* e);
 /* CudaQLearning::update_batch (src/q_learning.cu:108-174): n explicit
  * transitions on table `table` (0 for a shared table, the env index
  * otherwise).  All reads see the table as it was before the call; deltas that
- * hit the same (s,a) are summed in sample order and then applied.  Host arrays. */
+ * hit the same (s,a) are summed in sample order and then applied.  Host arrays.
+ * States outside the table are refused (CRL_E_RANGE); a sample whose action is
+ * outside [0, n_actions) changes nothing, as a step with such an action moves
+ * nothing (src/kernels.cu:15-23). */
 int crl_td_update(crl_engine* e, int32_t table, int32_t n, const int32_t* s, const int32_t* a,
                   const float* r, const int32_t* s_next, const uint8_t* done);
 

@@ -71,6 +71,32 @@ def test_create_rejects_bad_configs_without_touching_a_device(pycrl):
     assert lib.crl_destroy(None) == 0
 
 
+def test_host_only_entry_points_leave_an_error_text(pycrl):
+    """crl_last_error() names the calling thread's last failure also for the entry
+    points that touch no device (map generators, epsilon table, grid classifier)."""
+    lib = pycrl.load()
+    with pytest.raises(pycrl.CrlError, match="wall_frac") as e:
+        pycrl.gen_maps_noise(0, 2, 8, 8, 4, 1.5, 0.05, 10.0)
+    assert e.value.code == -1
+    with pytest.raises(pycrl.CrlError, match="one shared map or one map per env"):
+        pycrl.gen_maps_bernoulli(0, 3, 7, 4, 4, 0.1)
+    with pytest.raises(pycrl.CrlError, match="2 to 2\\^30 cells"):
+        pycrl.gen_maps_bernoulli(0, 1, 1, 1, 1, 0.1)
+    cfg = pycrl.make_config(4, 4, 4, eps_mode=1, eps_span=0)
+    n = C.c_int32()
+    assert lib.crl_eps_table(C.byref(cfg), None, 0, C.byref(n)) == -1
+    assert b"eps_span" in lib.crl_last_error()
+    assert lib.crl_classify_grid(None, 4, C.c_float(-0.01), None, None) == -1
+    assert b"crl_classify_grid" in lib.crl_last_error()
+    # another thread's failures are its own
+    import threading
+    seen = []
+    t = threading.Thread(target=lambda: seen.append(lib.crl_last_error()))
+    t.start()
+    t.join()
+    assert seen == [b""]
+
+
 def test_engine_fails_loudly_without_a_device(pycrl):
     """No CPU fallback: on a box without a HIP device crl_create reports
     CRL_E_DEVICE (on a GPU box this test has nothing to check)."""
@@ -237,6 +263,28 @@ def test_npy_agent_files_match_numpy(pycrl, tmp_path):
         cudarl_core.load_agent_npy(path, W, H, A)
     with pytest.raises(RuntimeError):
         cudarl_core.load_agent_npy(str(tmp_path / "missing.npy"), W, H, A)
+    # a header that promises more than the file holds is refused before anything is allocated
+    def write_npy(shape_text, payload):
+        head = "{'descr': '<f8', 'fortran_order': False, 'shape': %s, }" % shape_text
+        head += " " * ((64 - (10 + len(head) + 1) % 64) % 64) + "\n"
+        with open(path, "wb") as f:
+            f.write(b"\x93NUMPY\x01\x00" + len(head).to_bytes(2, "little") + head.encode() + payload)
+    payload = table.tobytes()
+    write_npy("(%d, %d, %d)" % (W, H, A), payload)
+    assert np.array_equal(np.load(path), table)  # the helper writes what numpy reads
+    assert np.array_equal(cudarl_core.load_agent_npy(path, W, H, A), got)
+    write_npy("(%d, %d, %d)" % (W, H, A), payload[:-8])
+    with pytest.raises(RuntimeError, match="truncated"):
+        cudarl_core.load_agent_npy(path, W, H, A)
+    write_npy("(%d, %d, %d)" % (W, H, 4000000000000000), payload)
+    with pytest.raises(RuntimeError, match="truncated"):
+        cudarl_core.load_agent_npy(path, W, H, A)
+    write_npy("(%d, %d, %d)" % (1 << 62, 1 << 62, 16), payload)  # the element count wraps around 2^64
+    with pytest.raises(RuntimeError, match="truncated"):
+        cudarl_core.load_agent_npy(path, W, H, A)
+    write_npy("(%d, %d, %d)" % (W, -H, A), payload)
+    with pytest.raises(RuntimeError, match="negative"):
+        cudarl_core.load_agent_npy(path, W, H, A)
     # raw fp32 tables of any shape
     big = rng.normal(0, 1, (3, 6, 8)).astype(np.float32)
     cudarl_core.save_table_npy(path, big)

@@ -565,6 +565,32 @@ def _td_case(gpu, oracle, W, H, A, s, a, r, s2, done, mode=0):
     assert_q_close(got.reshape(-1), want)
 
 
+def test_td_update_skips_samples_with_an_action_outside_the_table(gpu, oracle):
+    """An action that is no action moves nothing in a step (src/kernels.cu:15-23) and
+    has no table entry: such a sample changes nothing, the samples around it keep
+    their place in the order of the sums (one block of 256 samples: plain left to
+    right, so leaving the skipped samples out altogether gives the same bits)."""
+    W, H, A, n = 6, 5, 4, 250
+    rng = np.random.default_rng(42)
+    s, s2 = rng.integers(0, W * H, n), rng.integers(0, W * H, n)
+    a = rng.integers(0, A, n)
+    bad = rng.random(n) < 0.3
+    a[bad] = rng.choice([-1, A, A + 3, 100, -7], bad.sum())
+    r = rng.normal(0, 1, n).astype(np.float32)
+    done = (rng.random(n) < 0.2).astype(np.uint8)
+    _td_case(gpu, oracle, W, H, A, s, a, r, s2, done)
+    # the same table from the valid samples alone
+    cfg = gpu.make_config(1, W, H, table_mode=gpu.TABLE_SHARED, map_mode=gpu.MAP_SHARED)
+    Q0 = np.random.default_rng(W * H).normal(0, 1, (W * H, A)).astype(np.float32)
+    got = []
+    for keep in (np.ones(n, bool), ~bad):
+        with gpu.Engine(cfg, 0) as eng:
+            eng.q_set(0, Q0)
+            eng.td_update(0, s[keep], a[keep], r[keep], s2[keep], done[keep])
+            got.append(eng.q_get(0))
+    assert np.array_equal(got[0], got[1])
+
+
 def test_td_update_many_blocks_and_tiles(gpu, oracle):
     """70 000 samples = 274 blocks: more than one 256-block tile and 18 groups;
     deltas of mixed magnitude make a wrong association visible."""
