@@ -115,7 +115,7 @@ class HipEvents:
             self.hip.hipEventDestroy(e)
 
 
-def time_gpu(key, reps, warm_reps, launch_steps=None, n_override=None, resident=0, variant=0):
+def time_gpu(key, reps, warm_reps, launch_steps=None, n_override=None, resident=0, variant=0, clocks=False):
     """`reps` timed passes of `launch_steps` env-steps per env (default: the
     workload's own length) after `warm_reps` untimed ones."""
     wl = WORKLOADS[key]
@@ -148,13 +148,32 @@ def time_gpu(key, reps, warm_reps, launch_steps=None, n_override=None, resident=
         split = eng.fused_split()
         q_probe = eng.q_get(0)
         phases = None
-        if variant == 2 and cfg.table_mode == pycrl.TABLE_SHARED and info["name"].startswith("k_shared_persist"):
-            # clocks of the LAST launch, first workgroup; scaled to that launch's measured time
+        if clocks and cfg.table_mode == pycrl.TABLE_SHARED and info["name"].startswith("k_shared_persist"):
+            # one more launch, untimed above, of the instantiation that keeps phase clocks
+            # (first workgroup), scaled to that launch's own duration
+            eng.set_persist_clocks(True)
+            a, b = ev.new(), ev.new()
+            ev.record(a)
+            eng.run_fused(per)
+            ev.record(b)
+            eng.sync()
             clk = eng.persist_clocks()[0].astype(float)
-            names = ("wait_for_owners", "act", "block_sums", "drain_publish", "wait_for_blocks", "cells_to_tile",
-                     "tile_sums_publish", "loop")
-            us = rep_ms[-1] * 1e3 / per
-            phases = {k: us * c / clk.sum() for k, c in zip(names, clk)}
+            names = ("prepare_step", "wait_for_table", "select_move_delta", "block_sums_cells", "clear_tile",
+                     "wait_for_cells", "tile_sums_publish", "loop")
+            us = ev.elapsed_ms(a, b) * 1e3 / per
+            ev.free([a, b])
+            phases = {k: us * c / clk[:8].sum() for k, c in zip(names, clk[:8])}
+            phases["us_per_step_with_clocks"] = us
+            phases["polls_per_step_for_table"] = clk[8] / per
+            phases["polls_per_step_for_cells"] = clk[9] / per
+            # when each workgroup passed each mark of the middle step, in us after the first
+            # workgroup passed mark 7 (loop top): min / median / max over the workgroups
+            stamps = eng.persist_stamps[:info["grid"]].astype(np.int64)
+            stamps = (stamps - stamps[:, 7].min()) * 0.01
+            marks = [("loop_top", 7)] + [("after_" + names[i], i) for i in (0, 1, 2, 3, 4, 5, 6)]
+            phases["middle_step_marks_us_min_med_max"] = {
+                n: [round(float(np.min(stamps[:, i])), 2), round(float(np.median(stamps[:, i])), 2),
+                    round(float(np.max(stamps[:, i])), 2)] for n, i in marks}
     dev_ms = sum(rep_ms)
     secs = max(wall, dev_ms * 1e-3)
     return dict(n=n, launch_steps=per, reps=reps, env_steps=n * per * reps, steps_per_s=n * per * reps / secs,
@@ -288,6 +307,8 @@ def main():
                     help="only run one plain copy kernel of this many MiB (calibrates rocprofv3 counters)")
     ap.add_argument("--probe-barrier", action="store_true",
                     help="only measure barriers over co-resident workgroups built from device-scope loads and stores")
+    ap.add_argument("--clocks", action="store_true",
+                    help="shared table, one-launch kernel: one more launch with its phase clocks armed")
     ap.add_argument("--no-cpu", action="store_true", help="skip the cpu_baseline leg")
     ap.add_argument("--no-also", action="store_true", help="skip the side measurements of the other configs")
     args = ap.parse_args()
@@ -311,7 +332,7 @@ def main():
         return
     key = args.workload
     wl = WORKLOADS[key]
-    g = time_gpu(key, args.steps, args.warmup, args.launch_steps, args.envs, args.resident, args.variant)
+    g = time_gpu(key, args.steps, args.warmup, args.launch_steps, args.envs, args.resident, args.variant, args.clocks)
 
     per_launch_units = g["n"] * g["launch_steps"]
     bytes_per_launch = per_launch_units * wl["bytes"]

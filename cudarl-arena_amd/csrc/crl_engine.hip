@@ -79,15 +79,15 @@ struct DevBuf {
 };
 
 // Scratch of crl_run_fused_noalloc: one array per GPU, part of the loaded code
-// object, so the entry point never allocates.  Layout: 4 KB of counters (ticket
-// counters at 0, the one-launch shared-table kernel's step flags at 1 KB and its
-// give-up word at 3 KB), then the hand-off cells of the ordered reduction.  The array's name
+// object, so the entry point never allocates.  Layout: 4 KB of counters (the ticket
+// counters), then 10 MB for what the workgroups of a shared-table step exchange: the
+// hand-off cells of the ordered reduction, or all exchange buffers of the one-launch
+// kernel.  The array's name
 // is a host-side stand-in, not a device address: host code only ever uses the
 // address hipGetSymbolAddress returned for the device at hand.
 constexpr size_t kScratchTicketBytes = 4096;
-constexpr size_t kScratchFlagsAt = 1024, kScratchErrAt = 3072;
-constexpr size_t kScratchHandoffBytes = (size_t)8 << 20;
-constexpr size_t kScratchBytes = kScratchTicketBytes + kScratchHandoffBytes;
+constexpr size_t kScratchExchangeBytes = (size_t)10 << 20;
+constexpr size_t kScratchBytes = kScratchTicketBytes + kScratchExchangeBytes;
 static __device__ __align__(256) unsigned char scratch[kScratchBytes];
 
 constexpr int kMaxDevices = 64;
@@ -132,14 +132,18 @@ struct crl_engine {
   bool no_alloc = false;
   unsigned char* static_scratch = nullptr;
   unsigned* tk = nullptr;  // ticket counters {next ticket, envs on HBM tables, envs on LDS tables}
-  uint2* ho = nullptr;     // hand-off cells of the ordered reduction
-  // one-launch shared-table kernel: step flags + give-up word, and whether a launch
-  // has not been checked for having given up yet
-  DevBuf<unsigned> pflags;
-  unsigned* perr = nullptr;
+  unsigned long long* ho = nullptr;  // hand-off cells of the ordered reduction
+  // one-launch shared-table kernel: what its workgroups exchange (tagged table, row
+  // maxima, marks, raw samples, hand-off cells), the engine's own give-up word
+  // followed by the phase clocks, and whether a launch has not been checked for
+  // having given up yet
+  DevBuf<unsigned long long> pbuf;
+  DevBuf<unsigned long long> pdiag;  // [0] give-up word, [1..16] phase clocks; allocated at crl_create
   bool persist_unchecked = false;
+  bool persist_failed = false;   // a launch gave up: state and table are not valid until they are set again
   bool persist_refused = false;  // the device refused the co-resident launch once: not tried again
-  int persist_spin_limit = crl::kPersistSpinLimit;  // polls a workgroup waits for its peers before it gives up
+  bool persist_clocks = false;   // run the instantiation that keeps phase clocks
+  int persist_spin_limit = crl::kPersistSpinLimit;  // polls a thread waits for its peers before it gives up
 
   DevBuf<int32_t> s, ep_step, episode, start, act;
   DevBuf<float> reward;
@@ -162,7 +166,7 @@ struct crl_engine {
   // first pass hands to the key owners
   DevBuf<int32_t> key;
   DevBuf<float> delta;
-  DevBuf<uint2> handoff;
+  DevBuf<unsigned long long> handoff;
   bool lds_opt_in = false;
   // scratch of crl_td_update
   DevBuf<int32_t> b_s, b_a, b_s2;
@@ -283,7 +287,9 @@ struct FusedPlan {
 };
 
 constexpr size_t kLdsPerWorkgroup = 160 * 1024;  // gfx950
-constexpr size_t kPersistStaticLds = 1024;      // static LDS of the one-launch shared-table kernel, rounded up
+// static LDS of kernels that call the workgroup-wide "or" (the device library keeps a few
+// words there), rounded up: their dynamic LDS can be at most the rest
+constexpr size_t kStaticLdsReserve = 1024;
 
 // Launches shorter than this do not repay moving whole tables into LDS and back
 // (1M envs of config 4, steps per launch -> env-steps/s, plain / hybrid:
@@ -496,7 +502,7 @@ int ceil_log2(size_t v) {
 crl::ReduceGeom reduce_geom(const crl_engine* e, int n) {
   crl::ReduceGeom G{};
   G.K = (int)e->K;
-  G.key_bits = std::max(1, ceil_log2(e->K));
+  G.a_shift = e->A == 8 ? 3 : 2;
   G.own_shift = ceil_log2((e->K + crl::kOwnKeys - 1) / crl::kOwnKeys);
   G.n_blocks = (n + crl::kBlockSamples - 1) / crl::kBlockSamples;
   return G;
@@ -526,25 +532,35 @@ int opt_in_lds(crl_engine* e) {
   const size_t act = kLdsPerWorkgroup;  // what a launch asks for is checked against this
   HIP_TRY(allow_lds(crl::k_reduce_blocks, sizeof(crl::ReduceLds)));
   HIP_TRY(allow_lds(crl::k_reduce_owners, kOwnersLds));
-  HIP_TRY(allow_lds(crl::k_shared_act<4, 1, true>, act));
-  HIP_TRY(allow_lds(crl::k_shared_act<4, 2, true>, act));
-  HIP_TRY(allow_lds(crl::k_shared_act<8, 1, true>, act));
-  HIP_TRY(allow_lds(crl::k_shared_act<8, 2, true>, act));
-  HIP_TRY(allow_lds(crl::k_shared_persist<4, 1>, act - kPersistStaticLds));
-  HIP_TRY(allow_lds(crl::k_shared_persist<4, 2>, act - kPersistStaticLds));
-  HIP_TRY(allow_lds(crl::k_shared_persist<8, 1>, act - kPersistStaticLds));
-  HIP_TRY(allow_lds(crl::k_shared_persist<8, 2>, act - kPersistStaticLds));
+  HIP_TRY(allow_lds(crl::k_shared_act<4, 1, true>, act - kStaticLdsReserve));
+  HIP_TRY(allow_lds(crl::k_shared_act<4, 2, true>, act - kStaticLdsReserve));
+  HIP_TRY(allow_lds(crl::k_shared_act<8, 1, true>, act - kStaticLdsReserve));
+  HIP_TRY(allow_lds(crl::k_shared_act<8, 2, true>, act - kStaticLdsReserve));
+  HIP_TRY(allow_lds(crl::k_shared_persist<4, 1, false>, act - kStaticLdsReserve));
+  HIP_TRY(allow_lds(crl::k_shared_persist<4, 2, false>, act - kStaticLdsReserve));
+  HIP_TRY(allow_lds(crl::k_shared_persist<8, 1, false>, act - kStaticLdsReserve));
+  HIP_TRY(allow_lds(crl::k_shared_persist<8, 2, false>, act - kStaticLdsReserve));
+  HIP_TRY(allow_lds(crl::k_shared_persist<4, 1, true>, act - kStaticLdsReserve));
+  HIP_TRY(allow_lds(crl::k_shared_persist<4, 2, true>, act - kStaticLdsReserve));
+  HIP_TRY(allow_lds(crl::k_shared_persist<8, 1, true>, act - kStaticLdsReserve));
+  HIP_TRY(allow_lds(crl::k_shared_persist<8, 2, true>, act - kStaticLdsReserve));
   e->lds_opt_in = true;
   return CRL_OK;
 }
 
+// the hand-off cells fit where this call may keep them
+bool handoff_fits(const crl_engine* e, const crl::ReduceGeom& G) {
+  return !e->no_alloc || handoff_records(G) * sizeof(unsigned long long) <= kScratchExchangeBytes;
+}
+
 int ensure_handoff(crl_engine* e, const crl::ReduceGeom& G) {
-  const size_t recs = handoff_records(G);  // (G.n_blocks: blocks, or workgroups of the one-launch kernel)
+  const size_t recs = handoff_records(G);
   if (e->no_alloc) {
-    if (recs * sizeof(uint2) > kScratchHandoffBytes)
+    if (!handoff_fits(e, G))
       return fail(CRL_E_RANGE, "the ordered reduction of this engine needs %zu bytes of hand-off cells, "
-                  "the static scratch of crl_run_fused_noalloc holds %zu", recs * sizeof(uint2), kScratchHandoffBytes);
-    e->ho = reinterpret_cast<uint2*>(e->static_scratch + kScratchTicketBytes);
+                  "the static scratch of crl_run_fused_noalloc holds %zu", recs * sizeof(unsigned long long),
+                  kScratchExchangeBytes);
+    e->ho = reinterpret_cast<unsigned long long*>(e->static_scratch + kScratchTicketBytes);
   } else {
     hipError_t h = e->handoff.ensure(recs);
     if (h != hipSuccess) return fail(CRL_E_ALLOC, "hand-off buffer allocation failed: %s", hipGetErrorString(h));
@@ -607,7 +623,7 @@ int shared_step(crl_engine* e, uint64_t t, int trace_row) {
   // LDS each step measured slower than the row reads it saves (12.4 against 12.05 us
   // per step on 65,536 envs, also against the five speculative reads per env).
   size_t lds = fast ? sizeof(crl::ReduceLds) : 0;
-  const size_t limit = fast ? kLdsPerWorkgroup : (size_t)64 * 1024;
+  const size_t limit = fast ? kLdsPerWorkgroup - kStaticLdsReserve : (size_t)64 * 1024;
   const size_t map_bytes = (size_t)e->map_words * 4;
   const bool lds_map = e->cfg.map_mode == CRL_MAP_SHARED && map_bytes <= (size_t)kLdsMapLimitBytes &&
                        lds + map_bytes <= limit;
@@ -630,22 +646,26 @@ int shared_step(crl_engine* e, uint64_t t, int trace_row) {
 
 // ---- shared table: all steps of a call in one launch ---------------------------------
 
-struct PersistPlan {  // (kPersistStaticLds: the kernel's own static LDS, rounded up)
+struct PersistPlan {
   bool ok;
   int grid;
   bool lds_map;
   size_t lds;
   crl::ReduceGeom G;
+  // what the workgroups exchange, in 64-bit words from the start of one buffer
+  size_t at_table, at_rowmax, at_mark, at_raw, at_cells, words;
 };
+
+// Shortest call worth the set-up of the one-launch kernel (clearing what its workgroups
+// exchange, one co-resident launch) instead of two plain launches per step.
+constexpr int kPersistMinSteps = 4;
 
 // The one-launch kernel needs every workgroup resident at once (one per compute
 // unit), the dense LDS table of the block pass and one tile of the owners' pass.
 PersistPlan plan_persist(const crl_engine* e, int n_steps) {
   PersistPlan p{};
-  // Only on request: measured on 65,536 envs / 64x64x4 it takes 16 us per step against the
-  // 12 us of two launches per step - a barrier over 256 workgroups through memory costs
-  // 2.5 to 3 us however the flags are laid out, a kernel boundary 1.6 us.
-  if (e->cfg.table_mode != CRL_TABLE_SHARED || e->fused_variant != 2 || e->persist_refused) return p;
+  if (e->cfg.table_mode != CRL_TABLE_SHARED || e->fused_variant == 1 || e->persist_refused) return p;
+  if (e->fused_variant == 0 && n_steps < kPersistMinSteps) return p;
   const int n_blocks = (e->N + crl::kBlockSamples - 1) / crl::kBlockSamples;
   p.G = reduce_geom(e, e->N);
   const int n_own = 1 << p.G.own_shift;
@@ -653,28 +673,39 @@ PersistPlan plan_persist(const crl_engine* e, int n_steps) {
   if (e->K > (size_t)crl::kDenseKeys || p.grid > crl::kPersistMaxGroups || p.grid > kComputeUnits) return p;
   p.G.n_blocks = p.grid;  // workgroups without envs hand over empty cells
   const size_t map_bytes = (size_t)e->map_words * 4;
-  p.lds_map = e->cfg.map_mode == CRL_MAP_SHARED && crl::kPersistReduceLds + map_bytes <= kLdsPerWorkgroup - kPersistStaticLds;
-  p.lds = crl::kPersistReduceLds + (p.lds_map ? map_bytes : 0);
+  p.lds_map = e->cfg.map_mode == CRL_MAP_SHARED && sizeof(crl::PersistLds) + map_bytes <= kLdsPerWorkgroup - kStaticLdsReserve;
+  p.lds = sizeof(crl::PersistLds) + (p.lds_map ? map_bytes : 0);
+  auto pad = [](size_t words) { return (words + 31) & ~(size_t)31; };  // 256-byte pieces
+  p.at_table = 0;
+  p.at_rowmax = p.at_table + pad(e->K);
+  p.at_mark = p.at_rowmax + pad(e->S);
+  p.at_raw = p.at_mark + pad((size_t)n_own);
+  p.at_cells = p.at_raw + pad(2 * (size_t)e->N);  // raw samples and cells: two buffers each
+  p.words = p.at_cells + 2 * (size_t)n_own * p.grid * crl::kHandoffRecs;
+  if (e->no_alloc && p.words * sizeof(unsigned long long) > kScratchExchangeBytes) return p;
   p.ok = true;
   return p;
 }
 
-template <int A, int MAP>
-hipError_t launch_persist_kernel(crl_engine* e, const PersistPlan& p, int n_steps, unsigned* flags) {
+template <int A, int MAP, bool CLK>
+hipError_t launch_persist_kernel(crl_engine* e, const PersistPlan& p, unsigned long long* buf, uint64_t t0,
+                                 int n_steps, int trace_row0) {
   crl::Rules R = e->rules();
   crl::Ptrs P = e->ptrs();
-  uint64_t t0 = e->t;
-  int n = n_steps, trace_row0 = e->trace_cursor;
-  int32_t* key = e->key.p;
-  float* delta = e->delta.p;
   crl::ReduceGeom G = p.G;
-  uint2* handoff = e->ho;
-  unsigned* err = e->perr;
+  crl::PersistBufs B{};
+  B.table = buf + p.at_table;
+  B.rowmax = buf + p.at_rowmax;
+  B.mark = buf + p.at_mark;
+  B.raw = buf + p.at_raw;
+  B.cells = buf + p.at_cells;
+  B.err = reinterpret_cast<unsigned*>(e->pdiag.p);
+  B.clocks = e->pdiag.p + 1;
   int spin_limit = e->persist_spin_limit;
-  void* args[] = {&R, &P, &t0, &n, &trace_row0, &key, &delta, &G, &handoff, &flags, &err, &spin_limit};
+  void* args[] = {&R, &P, &t0, &n_steps, &trace_row0, &G, &B, &spin_limit};
   // a cooperative launch is refused unless all workgroups can be resident together,
   // which the kernel's waits rely on
-  return hipLaunchCooperativeKernel(reinterpret_cast<const void*>(&crl::k_shared_persist<A, MAP>), dim3(p.grid),
+  return hipLaunchCooperativeKernel(reinterpret_cast<const void*>(&crl::k_shared_persist<A, MAP, CLK>), dim3(p.grid),
                                     dim3(256), args, (unsigned)p.lds, e->stream);
 }
 
@@ -684,33 +715,43 @@ int run_persist(crl_engine* e, int n_steps, bool* launched) {
   *launched = false;
   const PersistPlan p = plan_persist(e, n_steps);
   if (!p.ok) return CRL_OK;
-  unsigned* flags;
+  int rc;
+  unsigned long long* buf;
   if (e->no_alloc) {
-    flags = reinterpret_cast<unsigned*>(e->static_scratch + kScratchFlagsAt);
-    e->perr = reinterpret_cast<unsigned*>(e->static_scratch + kScratchErrAt);
+    buf = reinterpret_cast<unsigned long long*>(e->static_scratch + kScratchTicketBytes);
   } else {
-    if (e->pflags.ensure(2 * crl::kPersistMaxGroups + 64) != hipSuccess)
-      return fail(CRL_E_ALLOC, "flag allocation failed");
-    flags = e->pflags.p;
-    e->perr = e->pflags.p + 2 * crl::kPersistMaxGroups;
+    if (e->pbuf.ensure(p.words) != hipSuccess) return fail(CRL_E_ALLOC, "allocation of the exchange buffers failed");
+    buf = e->pbuf.p;
   }
-  int rc = ensure_handoff(e, p.G);
+  rc = opt_in_lds(e);
   if (rc) return rc;
-  // flags and the give-up word start at zero (the word follows the flags in both layouts'
-  // fill: two fills keep the static layout's gap untouched)
-  hipLaunchKernelGGL(crl::k_fill_u32, dim3(2), dim3(256), 0, e->stream, flags, 0u, 2 * crl::kPersistMaxGroups);
-  hipLaunchKernelGGL(crl::k_fill_u32, dim3(1), dim3(64), 0, e->stream, e->perr, 0u, 1);
-  hipError_t h;
-  if (e->A == 4)
-    h = p.lds_map ? launch_persist_kernel<4, 1>(e, p, n_steps, flags) : launch_persist_kernel<4, 2>(e, p, n_steps, flags);
-  else
-    h = p.lds_map ? launch_persist_kernel<8, 1>(e, p, n_steps, flags) : launch_persist_kernel<8, 2>(e, p, n_steps, flags);
-  if (h != hipSuccess) {
-    (void)hipGetLastError();  // not resident all at once on this device: never mind, two launches per step
-    e->persist_refused = true;
-    return CRL_OK;
+  // The kernel's tags count the steps of one launch, so everything the workgroups
+  // exchange starts from tag 0 (a fill kernel, not a memset: a caller may record this),
+  // and a call longer than the tags allow goes out as several launches.
+  int done = 0;
+  while (done < n_steps) {
+    const int n = std::min(n_steps - done, crl::kPersistMaxSteps);
+    const size_t w32 = p.words * 2;
+    hipLaunchKernelGGL(crl::k_fill_u32, dim3((unsigned)((w32 + 255) / 256)), dim3(256), 0, e->stream,
+                       reinterpret_cast<unsigned*>(buf), 0u, (int)w32);
+    const uint64_t t0 = e->t + (uint64_t)done;
+    const int row0 = (int)std::min<long long>((long long)e->trace_cursor + done, e->trace_cap);
+    hipError_t h;
+#define CRL_PERSIST(A, MAP) \
+  (e->persist_clocks ? launch_persist_kernel<A, MAP, true>(e, p, buf, t0, n, row0) \
+                     : launch_persist_kernel<A, MAP, false>(e, p, buf, t0, n, row0))
+    if (e->A == 4) h = p.lds_map ? CRL_PERSIST(4, 1) : CRL_PERSIST(4, 2);
+    else h = p.lds_map ? CRL_PERSIST(8, 1) : CRL_PERSIST(8, 2);
+#undef CRL_PERSIST
+    if (h != hipSuccess) {
+      (void)hipGetLastError();
+      if (done > 0) return fail(CRL_E_DEVICE, "the one-launch shared-table kernel was refused after %d steps: %s", done, hipGetErrorString(h));
+      e->persist_refused = true;  // not resident all at once on this device: never mind, two launches per step
+      return CRL_OK;
+    }
+    e->persist_unchecked = true;
+    done += n;
   }
-  e->persist_unchecked = true;
   if (e->trace_n > 0) {
     const long long c = (long long)e->trace_cursor + n_steps;
     e->trace_cursor = c > e->trace_cap ? e->trace_cap : (int)c;
@@ -719,16 +760,38 @@ int run_persist(crl_engine* e, int n_steps, bool* launched) {
   return CRL_OK;
 }
 
-// After a synchronisation: did a one-launch kernel give up waiting for its peers?
+// Did a one-launch kernel give up waiting for its peers?  Called by the entry points
+// that synchronise; reports a give-up once.  The give-up word stays set on the device
+// (the kernel's later launches see it and return at once), and until the caller has set
+// state or table again every call that works on them fails (require_valid).
 int check_persist(crl_engine* e) {
   if (!e->persist_unchecked) return CRL_OK;
   e->persist_unchecked = false;
   unsigned gave_up = 0;
-  HIP_TRY(hipMemcpyAsync(&gave_up, e->perr, sizeof gave_up, hipMemcpyDeviceToHost, e->stream));
+  HIP_TRY(hipMemcpyAsync(&gave_up, e->pdiag.p, sizeof gave_up, hipMemcpyDeviceToHost, e->stream));
   HIP_TRY(hipStreamSynchronize(e->stream));
-  if (gave_up)
-    return fail(CRL_E_DEVICE, "the one-launch shared-table kernel gave up waiting for its workgroups "
-                "(were they all resident?); state and table are not valid - use crl_set_fused_variant(e, 1)");
+  if (!gave_up) return CRL_OK;
+  e->persist_failed = true;
+  return fail(CRL_E_DEVICE, "the one-launch shared-table kernel gave up waiting for its workgroups "
+              "(were they all resident?); state and table are not valid: set them again (crl_reset, "
+              "crl_set_state, crl_q_set) and use crl_set_fused_variant(e, 1)");
+}
+
+int require_valid(const crl_engine* e) {
+  if (e->persist_failed)
+    return fail(CRL_E_STATE, "a one-launch shared-table kernel gave up earlier: state and table are not valid "
+                "until crl_reset, crl_set_state or crl_q_set");
+  return CRL_OK;
+}
+
+// The caller sets state or table again.  A launch nobody has looked at yet is looked at
+// first (and a give-up reported by this call); a give-up already reported is history.
+int clear_persist_failure(crl_engine* e) {
+  int rc = check_persist(e);
+  if (rc) return rc;
+  if (!e->persist_failed) return CRL_OK;
+  HIP_TRY(hipMemsetAsync(e->pdiag.p, 0, sizeof(unsigned long long), e->stream));
+  e->persist_failed = false;
   return CRL_OK;
 }
 
@@ -753,6 +816,11 @@ int check_engine(const crl_engine* e) {
   hipError_t err = hipSetDevice(e->device);
   if (err != hipSuccess) return fail(CRL_E_DEVICE, "hipSetDevice(%d): %s", e->device, hipGetErrorString(err));
   return CRL_OK;
+}
+
+int check_usable(const crl_engine* e) {
+  int rc = check_engine(e);
+  return rc ? rc : require_valid(e);
 }
 
 // move codes of maps [first, first + count) from the class maps on the device
@@ -836,6 +904,7 @@ int create_engine(const crl_config* cfg, int device, crl_engine** out) {
   if (cfg->table_mode == CRL_TABLE_SHARED) {
     acc(e->key.alloc(N));
     acc(e->delta.alloc(N));
+    acc(e->pdiag.alloc(1 + crl::kPersistClockWords));
   }
   if (cfg->track_returns) {
     acc(e->ret_acc.alloc(N));
@@ -869,6 +938,7 @@ int create_engine(const crl_config* cfg, int device, crl_engine** out) {
   if ((h = hipMemsetAsync(e->done.p, 0, N, e->stream)) != hipSuccess) return bail(h, "clear");
   if ((h = hipMemsetAsync(e->action.p, 0, N, e->stream)) != hipSuccess) return bail(h, "clear");
   if ((h = hipMemsetAsync(e->map.p, 0, e->map.n * 4, e->stream)) != hipSuccess) return bail(h, "clear");
+  if (e->pdiag.p && (h = hipMemsetAsync(e->pdiag.p, 0, e->pdiag.n * 8, e->stream)) != hipSuccess) return bail(h, "clear");
   if (cfg->track_returns) {
     void* bufs[] = {e->ret_acc.p, e->ret_last.p, e->ret_sum.p, e->len_last.p, e->len_sum.p};
     for (void* b : bufs)
@@ -893,6 +963,8 @@ int create_engine(const crl_config* cfg, int device, crl_engine** out) {
 
 int reset_envs(crl_engine* e, int32_t first, int32_t count) {
   int rc = check_engine(e);
+  if (rc) return rc;
+  rc = clear_persist_failure(e);
   if (rc) return rc;
   if (first < 0 || count < 0 || (int64_t)first + count > e->N)
     return fail(CRL_E_RANGE, "env range [%d,%d) outside [0,%d)", first, first + count, e->N);
@@ -988,6 +1060,13 @@ int run_fused(crl_engine* e, int32_t n_steps, bool no_alloc) {
   if (n_steps < 0) return fail(CRL_E_ARG, "negative step count");
   if (n_steps == 0) return CRL_OK;
   if (no_alloc && !e->static_scratch) return fail(CRL_E_STATE, "the device's scratch array was not found at crl_create");
+  rc = require_valid(e);
+  if (rc) return rc;
+  // whichever way this call ends, later calls work with the engine's own buffers again
+  struct Restore {
+    crl_engine* e;
+    ~Restore() { e->no_alloc = false; }
+  } restore{e};
   e->no_alloc = no_alloc;
   if (e->cfg.table_mode == CRL_TABLE_PER_ENV) {
     const FusedPlan p = plan_fused(e, n_steps);
@@ -1023,7 +1102,6 @@ int run_fused(crl_engine* e, int32_t n_steps, bool no_alloc) {
       if (e->trace_n > 0 && e->trace_cursor < e->trace_cap) e->trace_cursor += 1;
     }
   }
-  e->no_alloc = false;
   e->t += (uint64_t)n_steps;
   e->have_transition = false;
   e->have_actions = false;
@@ -1079,7 +1157,7 @@ int crl_set_fused_variant(crl_engine* e, int32_t variant) {
 }
 
 int crl_get_fused_split(crl_engine* e, uint32_t* hbm_envs, uint32_t* lds_envs) {
-  int rc = check_engine(e);
+  int rc = check_usable(e);
   if (rc) return rc;
   unsigned v[3] = {0, 0, 0};
   if (e->tk) {
@@ -1111,7 +1189,7 @@ int crl_set_cell(crl_engine* e, int32_t map_index, int32_t cell, int32_t cell_cl
 int crl_reset(crl_engine* e, int32_t first, int32_t count) { return reset_envs(e, first, count); }
 
 int crl_step(crl_engine* e, const int32_t* actions) {
-  int rc = check_engine(e);
+  int rc = check_usable(e);
   if (rc) return rc;
   if (actions) {
     HIP_TRY(hipMemcpyAsync(e->act.p, actions, (size_t)e->N * 4, hipMemcpyHostToDevice, e->stream));
@@ -1130,7 +1208,7 @@ int crl_step(crl_engine* e, const int32_t* actions) {
 }
 
 int crl_select(crl_engine* e, int32_t* actions_out) {
-  int rc = check_engine(e);
+  int rc = check_usable(e);
   if (rc) return rc;
   const long long threads = (long long)e->N * e->A;
   const int grid = (int)((threads + 255) / 256);
@@ -1150,7 +1228,7 @@ int crl_select(crl_engine* e, int32_t* actions_out) {
 }
 
 int crl_update(crl_engine* e) {
-  int rc = check_engine(e);
+  int rc = check_usable(e);
   if (rc) return rc;
   if (!e->have_transition) return fail(CRL_E_STATE, "crl_update needs a preceding crl_step");
   const crl::Rules R = e->rules();
@@ -1183,7 +1261,7 @@ int crl_update(crl_engine* e) {
 
 int crl_td_update(crl_engine* e, int32_t table, int32_t n, const int32_t* s, const int32_t* a,
                   const float* r, const int32_t* s_next, const uint8_t* done) {
-  int rc = check_engine(e);
+  int rc = check_usable(e);
   if (rc) return rc;
   if (table < 0 || table >= e->n_tables) return fail(CRL_E_RANGE, "table %d outside [0,%d)", table, e->n_tables);
   if (n < 0) return fail(CRL_E_ARG, "negative sample count");
@@ -1233,7 +1311,7 @@ int crl_run_fused_noalloc(crl_engine* e, int32_t n_steps) { return run_fused(e, 
 
 int crl_get_state(crl_engine* e, int32_t* s, float* reward, uint8_t* done, uint8_t* action,
                   int32_t* ep_step, int32_t* episode) {
-  int rc = check_engine(e);
+  int rc = check_usable(e);
   if (rc) return rc;
   const size_t N = (size_t)e->N;
   if (s) HIP_TRY(hipMemcpyAsync(s, e->s.p, N * 4, hipMemcpyDeviceToHost, e->stream));
@@ -1248,6 +1326,8 @@ int crl_get_state(crl_engine* e, int32_t* s, float* reward, uint8_t* done, uint8
 
 int crl_set_state(crl_engine* e, const int32_t* s, const int32_t* ep_step, const int32_t* episode) {
   int rc = check_engine(e);
+  if (rc) return rc;
+  rc = clear_persist_failure(e);
   if (rc) return rc;
   const size_t N = (size_t)e->N;
   if (s) {
@@ -1265,7 +1345,7 @@ int crl_set_state(crl_engine* e, const int32_t* s, const int32_t* ep_step, const
 
 int crl_get_episode_stats(crl_engine* e, float* last_return, int32_t* last_length, float* return_sum,
                           int32_t* length_sum) {
-  int rc = check_engine(e);
+  int rc = check_usable(e);
   if (rc) return rc;
   if (!e->cfg.track_returns) return fail(CRL_E_STATE, "the engine was created without track_returns");
   const size_t b = (size_t)e->N * 4;
@@ -1290,7 +1370,7 @@ int crl_set_step_count(crl_engine* e, uint64_t t) {
 }
 
 int crl_q_get_range(crl_engine* e, int32_t first_table, int32_t count, float* out) {
-  int rc = check_engine(e);
+  int rc = check_usable(e);
   if (rc) return rc;
   if (!out) return fail(CRL_E_ARG, "out is null");
   if (first_table < 0 || count < 0 || (int64_t)first_table + count > e->n_tables)
@@ -1305,6 +1385,8 @@ int crl_q_get(crl_engine* e, int32_t table, float* out) { return crl_q_get_range
 
 int crl_q_set(crl_engine* e, int32_t table, const float* in) {
   int rc = check_engine(e);
+  if (rc) return rc;
+  rc = clear_persist_failure(e);
   if (rc) return rc;
   if (!in) return fail(CRL_E_ARG, "in is null");
   if (table < 0 || table >= e->n_tables) return fail(CRL_E_RANGE, "table %d outside [0,%d)", table, e->n_tables);
@@ -1340,7 +1422,7 @@ int crl_set_trace(crl_engine* e, int32_t n_envs, int32_t max_steps) {
 
 int crl_get_trace(crl_engine* e, int32_t n_steps, int32_t* s_next, uint8_t* action, float* reward,
                   uint8_t* done) {
-  int rc = check_engine(e);
+  int rc = check_usable(e);
   if (rc) return rc;
   if (n_steps < 0 || n_steps > e->trace_cursor)
     return fail(CRL_E_RANGE, "%d steps asked, %d recorded", n_steps, e->trace_cursor);
@@ -1440,15 +1522,26 @@ int crl_fused_plan_for_config(const crl_config* cfg, int32_t n_steps, char* name
   return CRL_OK;
 }
 
-// Tuning aid: per-phase shader clocks, summed over the steps of the last one-launch
-// shared-table call, of its first (out[0..7]) and last (out[8..15]) workgroup.
+// Diagnostics: arms (or disarms) the phase clocks of the one-launch shared-table kernel.
+// Armed, the instantiation that reads the shader clock eight times per step runs.
+int crl_set_persist_clocks(crl_engine* e, int32_t on) {
+  if (!e) return fail(CRL_E_ARG, "null engine");
+  e->persist_clocks = on != 0;
+  return CRL_OK;
+}
+
+// Diagnostics: per-phase shader clocks, summed over the steps of the last one-launch
+// shared-table launch that ran with the clocks armed, of its first (out[0..7]) and
+// last (out[8..15]) workgroup.
 int crl_get_persist_clocks(crl_engine* e, uint64_t* out16) {
   int rc = check_engine(e);
   if (rc) return rc;
   if (!out16) return fail(CRL_E_ARG, "out16 is null");
-  if (!e->perr) return fail(CRL_E_STATE, "no one-launch shared-table kernel has run on this engine");
+  if (!e->pdiag.p) return fail(CRL_E_STATE, "this engine has no shared table");
   HIP_TRY(hipStreamSynchronize(e->stream));
-  HIP_TRY(hipMemcpy(out16, e->perr + 8, 16 * sizeof(uint64_t), hipMemcpyDeviceToHost));
+  rc = check_persist(e);
+  if (rc) return rc;
+  HIP_TRY(hipMemcpy(out16, e->pdiag.p + 1, crl::kPersistClockWords * sizeof(uint64_t), hipMemcpyDeviceToHost));
   return CRL_OK;
 }
 

@@ -886,19 +886,18 @@ __global__ __launch_bounds__(256) void k_shared_act(const Rules R, const Ptrs P,
                                                      const int trace_row,
                                                      int32_t* __restrict__ key,
                                                      float* __restrict__ delta, const ReduceGeom G,
-                                                     uint2* __restrict__ handoff) {
-  extern __shared__ unsigned char lds_raw[];
+                                                     unsigned long long* __restrict__ handoff) {
+  extern __shared__ __align__(16) unsigned char lds_raw[];
   uint32_t* lds_map = reinterpret_cast<uint32_t*>(lds_raw + (REDUCE ? sizeof(ReduceLds) : 0));
   const int tid = threadIdx.x;
   const int env = blockIdx.x * blockDim.x + tid;
   bool live = env < P.N;
   // the env's cell is fetched while the map streams into LDS
   const int s_in = live ? P.s[env] : 0;
-  if (REDUCE) reduce_block_clear(*reinterpret_cast<ReduceLds*>(lds_raw), G);
-  if (MAP == 1) {
+  if (REDUCE) reduce_block_init(*reinterpret_cast<ReduceLds*>(lds_raw));
+  if (MAP == 1)
     for (int i = tid; i < P.map_words; i += blockDim.x) lds_map[i] = P.map[i];
-    __syncthreads();
-  }
+  if (MAP == 1 || REDUCE) __syncthreads();
   int my_key = 0;
   float my_delta = 0.0f;
   if (live && R.max_episodes > 0 && P.episode[env] >= R.max_episodes) {
@@ -985,7 +984,7 @@ __global__ __launch_bounds__(256) void k_shared_act(const Rules R, const Ptrs P,
   }
   if (REDUCE) {
     ReduceLds& L = *reinterpret_cast<ReduceLds*>(lds_raw);
-    reduce_block(L, G, blockIdx.x, my_key, my_delta, live, handoff);
+    reduce_block<false>(L, G, blockIdx.x, my_key, my_delta, live, handoff, 0u);
   }
 }
 

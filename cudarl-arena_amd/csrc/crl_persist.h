@@ -1,272 +1,146 @@
 // Shared table, all steps of a launch in ONE kernel: every workgroup is a block of
 // the ordered reduction (256 envs, state in registers for the whole launch) and
-// the owner of 64 keys, and the two roles hand their data to each other through
-// memory that is read and written past the caches' incoherent levels.
+// the owner of 64 keys (64 / A whole table rows, values in registers), and the two
+// roles hand their data to each other through memory.
 //
-// gfx950 has eight XCDs, each with its own L2; plain loads and stores are
-// coherent inside one XCD only, and the release / acquire fences that make them
-// coherent across the chip write back and invalidate a whole L2.  Loads and stores
-// carrying the `sc1` bit (device scope) are served past the L2: a value stored
-// that way by one workgroup is seen by the next sc1 load of any other (measured:
-// about 170 ns per dependent sc1 access, also between XCDs).  So everything the
-// workgroups exchange - the table, the hand-off cells, the (key, delta) arrays
-// and the step flags - is only ever touched with sc1 accesses inside this kernel,
-// and an exchange is: sc1 stores, wait until they are acknowledged, sc1 store of
-// the workgroup's flag; the reader polls the flags, then sc1-loads the data.
+// What is exchanged is only ever touched with device-scope accesses (st_dev64 /
+// ld_dev64: coherent between the eight XCDs without fences), and every exchanged
+// datum is a 64-bit unit that carries the tag of the step it belongs to.  A reader
+// asks for the data itself, again and again until the tags are the step's: there
+// are no flags, no "store, wait for the acknowledgement, then publish", and one
+// trip through memory per exchange instead of two.
 //
-// One step:
-//   1. wait until every owner has published the table of this step   (owner flags)
-//   2. act: select, move, (key, delta) from the table as published
-//   3. fold the block's deltas in order, hand the block sums to the owners'
-//      cells, publish                                                 (block flag)
-//   4. as owner: wait for every block's cells, add them in tree order, store
-//      the 64 new table values, publish                               (owner flag)
-// A workgroup writes its cells of step k+1 only after step 1 of k+1, when every
-// owner has consumed the cells of step k, and an owner overwrites its table values
-// only after step 4's wait, when every block has read them: one buffer of each.
+//   table[key]   {value, tag}   published by the key's owner
+//   rowmax[cell] {max of the row, tag}   by the owner of the row
+//   mark[owner]  {0, tag}       "this owner has consumed the cells of the step before" (read by workgroups that are no owners)
+//   cell[block][owner][8]       block sums, records as in crl_reduce.h; written whole every step
+//   raw[env]     {delta, key, tag}   only from blocks whose cell for some owner overflowed
 //
-// Every wait is bounded: a workgroup that waits for `spin_limit` polls (default
-// kPersistSpinLimit) sets the error word and leaves; the others then leave, too.
+// One step k (tag k + 1 for what the blocks read, k + 2 for the table that results):
+//   block:  what does not depend on the table (exploration draw, neighbour cells, move
+//           codes; the owner's stores are on their way meanwhile) -> poll own row and
+//           the A neighbours' row maxima -> select, move, (key, delta) -> ordered block
+//           sums -> cells
+//   owner:  clear the tile, wait until the cells are acknowledged -> poll the cells of
+//           all blocks -> tile -> sums in tree order -> new values, row maxima and mark
+// An owner overwrites its values only after it has every block's cells of the step,
+// which a block writes after all its threads have read theirs: one buffer of table
+// and row maxima suffices.  Cells and raw samples have two buffers, taken in turn: a
+// workgroup that writes the cells of step k + 2 has read table values of step k + 2,
+// so some owner has had the cells of step k + 1 of ALL workgroups, which - a
+// workgroup does its two roles one after the other - were all through with their
+// owner's part of step k by then.  That argument needs a workgroup to wait for table
+// values or, as an owner, for cells; a workgroup that is no owner (more blocks than
+// owners) might have no env left to wait for, so those poll every owner's mark
+// (one thread each) as well.
+//
+// Every wait is bounded: a thread that polls `spin_limit` times in vain (or sees the
+// give-up word set) makes its workgroup set the give-up word and leave.
 #pragma once
 #include "crl_kernels.h"
 
 namespace crl {
 
-constexpr int kPersistSpinLimit = 1 << 20;  // polls of about a quarter microsecond each
+constexpr int kPersistSpinLimit = 1 << 20;  // polls of a fraction of a microsecond each
 constexpr int kPersistMaxGroups = 256;      // workgroups: one per compute unit, all resident
-constexpr size_t kPersistReduceLds =
-    sizeof(ReduceLds) > (size_t)(kTileBlocks + kTileBlocks / kGroupBlocks) * kOwnKeys * sizeof(float)
-        ? sizeof(ReduceLds)
-        : (size_t)(kTileBlocks + kTileBlocks / kGroupBlocks) * kOwnKeys * sizeof(float);
+constexpr int kPersistMaxSteps = 65535;     // per launch: the raw samples' tags have 17 bits
+constexpr int kPersistTablePause = 4;       // x 128 clocks between a step's preparation and its first look at the table
+constexpr int kPersistClockWords = 20 + 8 * 256;  // 2 workgroups x (8 phases + polls of the two waits by thread 0),
+                                                  // then the wall clock of every workgroup at the 8 marks of one step
 
-// ---- device-scope (sc1) accesses -----------------------------------------------
-// Stores are fire-and-forget until drain_stores().  Loads come in groups that are
-// issued together and waited for inside ONE asm statement, with early-clobber
-// outputs: the compiler does not know that a load writes its destination later
-// and would otherwise reuse those registers while the load is in flight.
+struct alignas(16) PersistLds {
+  ReduceLds red;
+  alignas(16) float tile[kTileBlocks * kOwnKeys];       // the owner's [block][key] block sums (cleared 16 bytes at a time)
+  float gsum[(kTileBlocks / kGroupBlocks) * kOwnKeys];  // [group][key]
+  float o_delta[kBlockSamples];                         // raw samples of one overflowing block
+  uint8_t o_slot[kBlockSamples];
+  uint8_t o_list[kTileBlocks];  // blocks whose cell overflowed this step
+  int o_count;
+  int dead;  // some thread gave up waiting (never cleared)
+};
 
-__device__ __forceinline__ void st_dev(unsigned* p, unsigned v) {
-  asm volatile("global_store_dword %0, %1, off sc1" ::"v"(p), "v"(v) : "memory");
-}
-__device__ __forceinline__ void st_dev(int32_t* p, int32_t v) {
-  asm volatile("global_store_dword %0, %1, off sc1" ::"v"(p), "v"(v) : "memory");
-}
-__device__ __forceinline__ void st_dev(float* p, float v) {
-  asm volatile("global_store_dword %0, %1, off sc1" ::"v"(p), "v"(v) : "memory");
-}
-__device__ __forceinline__ void st_dev(uint2* p, uint2 v) {
-  asm volatile("global_store_dwordx2 %0, %1, off sc1" ::"v"(p), "v"(v) : "memory");
-}
-__device__ __forceinline__ void drain_stores() { asm volatile("s_waitcnt vmcnt(0)" ::: "memory"); }
+struct PersistBufs {
+  unsigned long long* table;   // [K]
+  unsigned long long* rowmax;  // [S]
+  unsigned long long* mark;    // [owners]
+  unsigned long long* cells;   // [owners][workgroups][8]
+  unsigned long long* raw;     // [N]
+  unsigned* err;               // give-up word
+  unsigned long long* clocks;  // kPersistClockWords phase clocks, or null
+};
 
-__device__ __forceinline__ unsigned ld_dev(const unsigned* p) {
-  unsigned v;
-  asm volatile("global_load_dword %0, %1, off sc1\n s_waitcnt vmcnt(0)" : "=&v"(v) : "v"(p) : "memory");
-  return v;
+__device__ __forceinline__ unsigned long long tagged(uint32_t bits, uint32_t tag) {
+  return (unsigned long long)bits | ((unsigned long long)tag << 32);
 }
-__device__ __forceinline__ uint4 ld_dev4(const uint4* p) {
-  uint4 v;
-  asm volatile("global_load_dwordx4 %0, %1, off sc1\n s_waitcnt vmcnt(0)" : "=&v"(v) : "v"(p) : "memory");
-  return v;
-}
-__device__ __forceinline__ void ld_dev4x2(const uint4* p0, const uint4* p1, uint4& v0, uint4& v1) {
-  asm volatile(
-      "global_load_dwordx4 %0, %2, off sc1\n global_load_dwordx4 %1, %3, off sc1\n s_waitcnt vmcnt(0)"
-      : "=&v"(v0), "=&v"(v1)
-      : "v"(p0), "v"(p1)
-      : "memory");
-}
-__device__ __forceinline__ void ld_dev4x4(const uint4* p0, const uint4* p1, const uint4* p2, const uint4* p3,
-                                          uint4& v0, uint4& v1, uint4& v2, uint4& v3) {
-  asm volatile(
-      "global_load_dwordx4 %0, %4, off sc1\n global_load_dwordx4 %1, %5, off sc1\n"
-      "global_load_dwordx4 %2, %6, off sc1\n global_load_dwordx4 %3, %7, off sc1\n s_waitcnt vmcnt(0)"
-      : "=&v"(v0), "=&v"(v1), "=&v"(v2), "=&v"(v3)
-      : "v"(p0), "v"(p1), "v"(p2), "v"(p3)
-      : "memory");
-}
-__device__ __forceinline__ void ld_dev4x5(const uint4* p0, const uint4* p1, const uint4* p2, const uint4* p3,
-                                          const uint4* p4, uint4& v0, uint4& v1, uint4& v2, uint4& v3,
-                                          uint4& v4) {
-  asm volatile(
-      "global_load_dwordx4 %0, %5, off sc1\n global_load_dwordx4 %1, %6, off sc1\n"
-      "global_load_dwordx4 %2, %7, off sc1\n global_load_dwordx4 %3, %8, off sc1\n"
-      "global_load_dwordx4 %4, %9, off sc1\n s_waitcnt vmcnt(0)"
-      : "=&v"(v0), "=&v"(v1), "=&v"(v2), "=&v"(v3), "=&v"(v4)
-      : "v"(p0), "v"(p1), "v"(p2), "v"(p3), "v"(p4)
-      : "memory");
-}
+__device__ __forceinline__ uint32_t tag_of(unsigned long long v) { return (uint32_t)(v >> 32); }
+__device__ __forceinline__ float value_of(unsigned long long v) { return __uint_as_float((uint32_t)v); }
 
-__device__ __forceinline__ float max4(const uint4 r) {
-  return fmaxf(fmaxf(__uint_as_float(r.x), __uint_as_float(r.y)), fmaxf(__uint_as_float(r.z), __uint_as_float(r.w)));
-}
+// raw sample: delta in the low word; key, valid bit and a 17-bit tag in the high word
+constexpr uint32_t kRawKeyMask = 0x3FFFu, kRawValid = 0x4000u;
+constexpr int kRawTagShift = 15;
+static_assert(kDenseKeys - 1 <= (int)kRawKeyMask, "raw samples hold 14-bit keys");
+static_assert(kPersistMaxSteps + 1 < (1 << (32 - kRawTagShift)), "raw tags must be unique within a launch");
+static_assert((uint32_t)kPersistMaxSteps + 1u <= kRecTagMask, "record tags must be unique within a launch");
 
-// row of cell `cell` of the shared table and the row maxima of the cells the A
-// actions lead to (`nb[i]`: neighbour cell, or the cell itself at the grid's edge)
 template <int A>
-__device__ __forceinline__ void load_rows_dev(const float* Q, int cell, const int (&nb)[A], Row<A>& row,
-                                              float (&nb_max)[A]);
+__device__ __forceinline__ Row<A> row_of_tagged(const unsigned long long (&v)[A]);
 template <>
-__device__ __forceinline__ void load_rows_dev<4>(const float* Q, int cell, const int (&nb)[4], Row<4>& row,
-                                                 float (&nb_max)[4]) {
-  const uint4* T = reinterpret_cast<const uint4*>(Q);
-  uint4 r, n0, n1, n2, n3;
-  ld_dev4x5(T + cell, T + nb[0], T + nb[1], T + nb[2], T + nb[3], r, n0, n1, n2, n3);
-  row = Row<4>{__uint_as_float(r.x), __uint_as_float(r.y), __uint_as_float(r.z), __uint_as_float(r.w)};
-  nb_max[0] = max4(n0);
-  nb_max[1] = max4(n1);
-  nb_max[2] = max4(n2);
-  nb_max[3] = max4(n3);
+__device__ __forceinline__ Row<4> row_of_tagged<4>(const unsigned long long (&v)[4]) {
+  return Row<4>{value_of(v[0]), value_of(v[1]), value_of(v[2]), value_of(v[3])};
 }
 template <>
-__device__ __forceinline__ void load_rows_dev<8>(const float* Q, int cell, const int (&nb)[8], Row<8>& row,
-                                                 float (&nb_max)[8]) {
-  const uint4* T = reinterpret_cast<const uint4*>(Q);  // a row is two 16-byte halves
-  uint4 a, b, c, d;
-  ld_dev4x2(T + 2 * cell, T + 2 * cell + 1, a, b);
-  row = Row<8>{__uint_as_float(a.x), __uint_as_float(a.y), __uint_as_float(a.z), __uint_as_float(a.w),
-               __uint_as_float(b.x), __uint_as_float(b.y), __uint_as_float(b.z), __uint_as_float(b.w)};
-#pragma unroll
-  for (int i = 0; i < 8; i += 2) {
-    ld_dev4x4(T + 2 * nb[i], T + 2 * nb[i] + 1, T + 2 * nb[i + 1], T + 2 * nb[i + 1] + 1, a, b, c, d);
-    nb_max[i] = fmaxf(max4(a), max4(b));
-    nb_max[i + 1] = fmaxf(max4(c), max4(d));
-  }
+__device__ __forceinline__ Row<8> row_of_tagged<8>(const unsigned long long (&v)[8]) {
+  return Row<8>{value_of(v[0]), value_of(v[1]), value_of(v[2]), value_of(v[3]),
+                value_of(v[4]), value_of(v[5]), value_of(v[6]), value_of(v[7])};
 }
 
-// Wave 0 polls the first `n` flags until all have reached `want` (or the limit is
-// hit, or another workgroup has given up); every thread returns the same answer.
-__device__ __forceinline__ bool wait_flags(const unsigned* flags, int n, unsigned want, unsigned* err,
-                                           int* lds_dead, const int spin_limit) {
-  if (threadIdx.x < 64) {
-    const int i0 = (int)threadIdx.x * 4;
-    bool ok = true;
-    if (i0 < n) {
-      int spins = 0;
-      for (;;) {
-        const uint4 v = ld_dev4(reinterpret_cast<const uint4*>(flags + i0));
-        ok = (int)(v.x - want) >= 0 && (i0 + 1 >= n || (int)(v.y - want) >= 0) &&
-             (i0 + 2 >= n || (int)(v.z - want) >= 0) && (i0 + 3 >= n || (int)(v.w - want) >= 0);
-        if (ok) break;
-        if (++spins >= spin_limit || ((spins & 255) == 0 && ld_dev(err) != 0u)) break;
-      }
-    }
-    if (!__all(ok) && threadIdx.x == 0) {
-      st_dev(err, 1u);
-      *lds_dead = 1;
-    }
-  }
-  __syncthreads();
-  return *lds_dead == 0;
-}
-
-// reduce_block() with the hand-off written for readers on other XCDs
-__device__ __forceinline__ void reduce_block_dev(ReduceLds& L, const ReduceGeom G, const int block,
-                                                 const int key, const float delta, const bool valid,
-                                                 uint2* handoff) {
-  const int tid = threadIdx.x;
-  const int lane = tid & 63;
-  const int wave = tid >> 6;
-  const int n_own = 1 << G.own_shift;
-  unsigned long long peers = __ballot(valid);
-  for (int b = 0; b < G.key_bits; ++b) {
-    const bool bit = (key >> b) & 1;
-    const unsigned long long m = __ballot(bit);
-    peers &= bit ? m : ~m;
-  }
-  const bool leader = valid && (peers & ((1ull << lane) - 1ull)) == 0ull;
-  const int owner = owner_of(key, G.own_shift);
-  bool first = false;
-  int slot = 0;
-  constexpr int kAhead = 8;
-  unsigned long long rest = leader ? peers : 0ull;
-  float ahead[kAhead];
-#pragma unroll
-  for (int i = 0; i < kAhead; ++i) {
-    const int j = rest ? __builtin_ctzll(rest) : lane;
-    const float dj = __shfl(delta, j);
-    ahead[i] = rest ? dj : 0.0f;
-    rest &= rest - 1ull;
-  }
-  __syncthreads();
-  for (int w = 0; w < 4; ++w) {
-    if (wave == w) {
-      float acc = 0.0f;
-      if (leader) {
-        first = L.seen[key] == 0;
-        acc = first ? 0.0f : L.run[key];
-      }
-#pragma unroll
-      for (int i = 0; i < kAhead; ++i) acc = acc + ahead[i];  // lane order = sample order
-      while (__ballot(rest != 0ull) != 0ull) {
-        const int j = rest ? __builtin_ctzll(rest) : lane;
-        const float dj = __shfl(delta, j);
-        if (rest) acc = acc + dj;
-        rest &= rest - 1ull;
-      }
-      if (leader) {
-        L.run[key] = acc;
-        L.seen[key] = 1;
-        if (first) slot = atomicAdd(&L.handed[owner], 1);
-      }
-    }
-    __syncthreads();
-  }
-  if (leader && first && slot < kSlotCap) {
-    const size_t at = ((size_t)owner * G.n_blocks + block) * kHandoffRecs + slot;
-    uint32_t tag = (uint32_t)(key >> G.own_shift);
-    if (slot == 0) {
-      const int c = L.handed[owner];
-      tag |= (uint32_t)(c > kSlotCap ? kSlotOverflow : c) << 8;
-    }
-    st_dev(handoff + at, make_uint2(tag, __float_as_uint(L.run[key])));
-  }
-  if (tid < n_own && L.handed[tid] == 0)
-    st_dev(handoff + ((size_t)tid * G.n_blocks + block) * kHandoffRecs, make_uint2(0u, 0u));
-}
-
-// Phase clocks: thread 0 of the first and the last workgroup add up the shader clocks
-// between the marks of a step and leave the sums behind the give-up word (16 x 64 bit),
-// for crl_get_persist_clocks.  Phases: 0 wait for the owners, 1 act, 2 block sums,
-// 3 drain + publish, 4 wait for the blocks, 5 cells into the tile, 6 tile sums + publish,
-// 7 loop overhead.
-#define CRL_MARK(i)                                   \
-  do {                                                \
-    const unsigned long long now_ = clock64();        \
-    phase_[i] += now_ - last_;                        \
-    last_ = now_;                                     \
+// Phase clocks (CLK only): thread 0 of the first and the last workgroup add up the shader
+// clocks between the marks of a step.  Phases: 0 work before the table is needed, 1 wait
+// for the table, 2 select / move / delta, 3 ordered block sums + cells, 4 clearing the
+// tile, 5 wait for the cells, 6 tile + sums + publish, 7 loop overhead.
+#define CRL_MARK(i)                                                                         \
+  do {                                                                                      \
+    if (CLK) {                                                                              \
+      const unsigned long long now_ = clock64();                                            \
+      phase_[i] += now_ - last_;                                                            \
+      last_ = now_;                                                                         \
+      if (k == n_steps / 2 && tid == 0 && B.clocks) B.clocks[20 + wg * 8 + (i)] = wall_clock64(); \
+    }                                                                                       \
   } while (0)
 
 // MAP = 1: the shared map staged in LDS; MAP = 2: maps read from global memory
 // (they do not change during a launch, so plain loads are fine).
 // G.n_blocks is the number of workgroups (blocks without envs hand over empty cells).
-// flags: [0, kPersistMaxGroups) block flags, [kPersistMaxGroups, 2 * kPersistMaxGroups)
-// owner flags, all zero at launch; err: the give-up word, zero at launch.
-template <int A, int MAP>
+// Everything in B holds tag 0 at launch (cleared by the host), *B.err is zero.
+template <int A, int MAP, bool CLK>
 __global__ __launch_bounds__(256) void k_shared_persist(const Rules R, const Ptrs P, const uint64_t t0,
                                                          const int n_steps, const int trace_row0,
-                                                         int32_t* key, float* delta, const ReduceGeom G,
-                                                         uint2* handoff, unsigned* flags, unsigned* err,
+                                                         const ReduceGeom G, const PersistBufs B,
                                                          const int spin_limit) {
-  extern __shared__ unsigned char lds_raw[];
-  ReduceLds& L = *reinterpret_cast<ReduceLds*>(lds_raw);
-  float* tile = reinterpret_cast<float*>(lds_raw);  // the owner's [block][key] tile reuses the block's table
-  float* gsum = tile + kTileBlocks * kOwnKeys;
-  uint32_t* lds_map = reinterpret_cast<uint32_t*>(lds_raw + kPersistReduceLds);
-  __shared__ int lds_dead;
+  extern __shared__ __align__(16) unsigned char lds_raw[];
+  PersistLds& L = *reinterpret_cast<PersistLds*>(lds_raw);
+  static_assert(sizeof(PersistLds) % 16 == 0 && offsetof(PersistLds, tile) % 16 == 0, "16-byte LDS accesses");
+  uint32_t* lds_map = reinterpret_cast<uint32_t*>(lds_raw + sizeof(PersistLds));
   const int tid = threadIdx.x;
   const int lane = tid & 63;
   const int wave = tid >> 6;
   const int wg = blockIdx.x;
   const int env = wg * 256 + tid;
   const bool has_env = env < P.N;
-  const int n_groups = (int)gridDim.x;  // every workgroup publishes a block flag
-  const int n_own = 1 << G.own_shift;   // workgroups [0, n_own) are owners, too
+  const int n_own = 1 << G.own_shift;  // workgroups [0, n_own) are owners, too
   const bool is_owner = wg < n_own;
-  unsigned* block_flags = flags;
-  unsigned* owner_flags = flags + kPersistMaxGroups;
 
-  if (tid == 0) lds_dead = 0;
+  // a launch of this engine gave up earlier and nobody has set state and table again:
+  // nothing to do (the word is read once, so that all threads take the same way)
+  if (tid == 0) L.o_count = (int)ld_dev32(B.err);
+  __syncthreads();
+  if (L.o_count != 0) return;
+  __syncthreads();
+  reduce_block_init(L.red);
+  if (tid == 0) {
+    L.o_count = 0;
+    L.dead = 0;
+  }
   if (MAP == 1)
     for (int i = tid; i < P.map_words; i += 256) lds_map[i] = P.map[i];
   // env state lives in registers for the whole launch
@@ -279,62 +153,163 @@ __global__ __launch_bounds__(256) void k_shared_persist(const Rules R, const Ptr
   const int start = has_env ? P.start[env] : 0;
   const bool track = P.ret_acc != nullptr;
   float ret = (track && has_env) ? P.ret_acc[env] : 0.0f;
-  // owner: lane l of wave 0 keeps the table value of its key in a register
-  const int own_key = key_of(wg, lane, G.own_shift);
-  const bool own_live = is_owner && wave == 0 && own_key < G.K;
-  float q_own = own_live ? __uint_as_float(ld_dev(reinterpret_cast<const unsigned*>(P.Q + own_key))) : 0.0f;
   const uint32_t* gmap = P.map + ((P.map_shared || !has_env) ? 0 : (size_t)env * P.map_words);
   const float* cr = P.cell_reward ? P.cell_reward + ((P.map_shared || !has_env) ? 0 : (size_t)env * P.S) : nullptr;
+  const DevWindow w_table = dev_window(B.table), w_cells = dev_window(B.cells);
+  const size_t cells_half = (size_t)n_own * G.n_blocks * kHandoffRecs;  // 64-bit words of one buffer of cells
+  const bool cells_flag = (R.reward_flags & 1) != 0;
+  const bool base_cells = cells_flag && (R.reward_flags & 2) != 0;
+
+  // owner: lane l of wave 0 keeps the table value of its key in a register; the A lanes
+  // of a row sit side by side, the first of them also publishes the row's maximum
+  const int own_key = key_of(wg, lane, G);
+  const bool own_live = is_owner && wave == 0 && own_key < G.K;
+  float q_own = own_live ? P.Q[own_key] : 0.0f;
+  auto publish = [&](uint32_t tag) {  // wave 0 of an owner
+    float qs[A];
+#pragma unroll
+    for (int i = 0; i < A; ++i) qs[i] = __shfl(q_own, (lane & ~(A - 1)) + i);
+    if (own_live) {
+      st_dev64(B.table + own_key, tagged(__float_as_uint(q_own), tag));
+      if ((lane & (A - 1)) == 0) {
+        Row<A> row;
+        if constexpr (A == 4) row = Row<4>{qs[0], qs[1], qs[2], qs[3]};
+        else row = Row<8>{qs[0], qs[1], qs[2], qs[3], qs[4], qs[5], qs[6], qs[7]};
+        st_dev64(B.rowmax + (own_key >> G.a_shift), tagged(__float_as_uint(row_max(row, false, 0)), tag));
+      }
+    }
+    if (lane == 0) st_dev64(B.mark + wg, tagged(0u, tag));
+  };
+  if (is_owner && wave == 0) publish(1u);
   __syncthreads();
 
-  unsigned long long phase_[8] = {0, 0, 0, 0, 0, 0, 0, 0};
-  unsigned long long last_ = clock64();
-  for (int k = 0; k < n_steps; ++k) {
+  // What a step needs that does not depend on the table: computed for step k + 1 while
+  // the cells of step k are on their way to the owners.
+  bool live = false;
+  int s0 = 0, cls0 = kFree;
+  int nb[A];
+  uint32_t mv = 0;
+  Draw d{0.0f, 0};
+  float eps = 0.0f;
+  auto prepare = [&](int k) {
     const uint64_t t = t0 + (uint64_t)k;
-    CRL_MARK(7);
-    // 1. the table of this step: every owner has published its values of step k
-    if (k > 0 && !wait_flags(owner_flags, n_own, (unsigned)k, err, &lds_dead, spin_limit)) break;
-    CRL_MARK(0);
-    reduce_block_clear(L, G);
-
-    // 2. act
-    const bool live = has_env && !(R.max_episodes > 0 && episode >= R.max_episodes);
-    int my_key = 0;
-    float my_delta = 0.0f;
+    live = has_env && !(R.max_episodes > 0 && episode >= R.max_episodes);
     if (has_env && !live) trace_idle(P, env, trace_row0 + k, s);
+    s0 = s;
+    const int x0 = s0 % R.W, y0 = s0 / R.W;
     if (live) {
-      auto cls = [&](int cell) -> int {
-        const uint32_t word = (MAP == 1) ? lds_map[cell >> 4] : gmap[cell >> 4];
-        return cell_class_of(word, cell);
-      };
-      const int s0 = s;
-      int x = s0 % R.W, y = s0 / R.W;
-      int nb[A];
 #pragma unroll
       for (int i = 0; i < A; ++i) {
         int dx, dy;
         action_delta(i, A, dx, dy);
-        const bool in = (unsigned)(x + dx) < (unsigned)R.W && (unsigned)(y + dy) < (unsigned)R.H;
+        const bool in = (unsigned)(x0 + dx) < (unsigned)R.W && (unsigned)(y0 + dy) < (unsigned)R.H;
         nb[i] = in ? s0 + dy * R.W + dx : s0;
       }
-      Row<A> row;
-      float nb_max[A];
-      load_rows_dev<A>(P.Q, s0, nb, row, nb_max);
-      Draw d = pick_draw(explore_block(R.seed, (uint32_t)env, t >> 1), t, A);
+      auto word_of = [&](int w) -> uint32_t { return (MAP == 1) ? lds_map[w] : gmap[w]; };
+      mv = moves_of_cell<A>(word_of, R.W, R.H, x0, y0, s0);
+      cls0 = cell_class_of(word_of(s0 >> 4), s0);
+      d = pick_draw(explore_block(R.seed, (uint32_t)env, t >> 1), t, A);
       if (P.u_sup && t >= P.sup_t0 && t - P.sup_t0 < (uint64_t)P.sup_n) {
         const size_t o = (size_t)(t - P.sup_t0) * P.N + env;
         d.u = P.u_sup[o];
         d.a = P.a_sup[o];
       }
-      const float eps = eps_of(R, P.eps_tab, t, episode);
-      const int a = (d.u < eps) ? d.a : row_argmax(row);
-      bool hit;
-      step_rule(R, ClassRewards{R.step_reward, R.goal_reward, R.trap_reward}, cls, cr, x, y, a, reward, hit);
-      const int s2 = y * R.W + x;
-      done = hit || (!R.auto_reset && done);
-      float m = row_max(row, false, 0);  // the env stayed where it was
+      eps = eps_of(R, P.eps_tab, t, episode);
+    } else {
 #pragma unroll
-      for (int i = 0; i < A; ++i) m = (s2 != s0 && a == i) ? nb_max[i] : m;
+      for (int i = 0; i < A; ++i) nb[i] = 0;
+    }
+  };
+
+  unsigned long long phase_[10] = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
+  unsigned long long last_ = CLK ? clock64() : 0ull;
+  bool gave_up = false;
+  for (int k = 0; k < n_steps; ++k) {
+    const uint32_t want = (uint32_t)k + 1u;
+    CRL_MARK(7);
+    // (the values this workgroup published as an owner are on their way meanwhile)
+    prepare(k);
+    reduce_stage_init(reinterpret_cast<unsigned long long*>(L.tile), G, want);
+    // A first look that comes too early costs a whole round trip more than one that comes
+    // just in time: the values published at the end of the last step need about 1.5 us to
+    // be visible, the preparation above takes 1 us (65,536 envs on 64x64x4, us per step by
+    // pause: none 8.16, 4 x 128 clocks 7.78, 6 x 7.85, 8 x 7.91, 16 x 8.55).
+    for (int i = 0; i < kPersistTablePause; ++i) __builtin_amdgcn_s_sleep(2);
+    CRL_MARK(0);
+
+
+    // ---- the table of this step: own row, the neighbours' maxima, one owner's mark --
+    unsigned long long rq[A], rn[A];
+    {
+      const uint32_t qrow = (uint32_t)s0 * (uint32_t)(A * 8);  // byte offset of the row in the table
+      bool ok = false;
+      int spins = 0;
+      while (!ok) {
+        poll_fence();
+        unsigned long long mk = tagged(0u, want);
+        if (!is_owner && tid < n_own) mk = ld_dev64(B.mark + tid);
+        if (live) {
+#pragma unroll
+          for (int i = 0; i < A; ++i) rn[i] = ld_dev64(B.rowmax + nb[i]);
+          // the row: two values to a 16-byte load
+          const uint4 r0 = ld_dev128(w_table, qrow), r1 = ld_dev128(w_table, qrow + 16);
+          if constexpr (A == 8) {
+            const uint4 r2 = ld_dev128(w_table, qrow + 32), r3 = ld_dev128(w_table, qrow + 48);
+            rq[4] = tagged(r2.x, r2.y);
+            rq[5] = tagged(r2.z, r2.w);
+            rq[6] = tagged(r3.x, r3.y);
+            rq[7] = tagged(r3.z, r3.w);
+          }
+          rq[0] = tagged(r0.x, r0.y);
+          rq[1] = tagged(r0.z, r0.w);
+          rq[2] = tagged(r1.x, r1.y);
+          rq[3] = tagged(r1.z, r1.w);
+        }
+        ok = tag_of(mk) == want;
+        if (live) {
+#pragma unroll
+          for (int i = 0; i < A; ++i) ok = ok && tag_of(rq[i]) == want && tag_of(rn[i]) == want;
+        }
+        if (!ok && (++spins >= spin_limit || ((spins & 63) == 0 && ld_dev32(B.err) != 0u))) {
+          L.dead = 1;
+          break;
+        }
+      }
+      if (CLK) phase_[8] += (unsigned long long)spins + 1ull;
+      __syncthreads();
+      if (L.dead) {
+        gave_up = true;
+        break;
+      }
+    }
+    CRL_MARK(1);
+
+    // ---- select, move, (key, delta) ---------------------------------------------------
+    int my_key = 0;
+    float my_delta = 0.0f;
+    if (live) {
+      const Row<A> row = row_of_tagged<A>(rq);
+      const int a = (d.u < eps) ? d.a : row_argmax(row);
+      // the rule of step_rule() on the move code of the action: the class of the target
+      // cell, or kWall outside the grid
+      const int code = (int)((mv >> (2 * a)) & 3u);
+      int tgt = nb[0];
+      float m_tgt = value_of(rn[0]);
+#pragma unroll
+      for (int i = 1; i < A; ++i) {
+        tgt = (a == i) ? nb[i] : tgt;
+        m_tgt = (a == i) ? value_of(rn[i]) : m_tgt;
+      }
+      const bool moved = code < kTrap;
+      const bool trap = code == kTrap;
+      const int s2 = moved ? tgt : s0;
+      const bool hit = R.goal_mode == 0 ? code == kGoal : ((moved ? code : cls0) == kGoal);
+      const float by_class = hit ? R.goal_reward : trap ? R.trap_reward : R.step_reward;
+      float by_cell = 0.0f;
+      if (cells_flag) by_cell = cr[(trap && !hit) ? tgt : s2];
+      reward = (cells_flag && (hit || trap || base_cells)) ? by_cell : by_class;
+      done = hit || (!R.auto_reset && done);
+      float m = (s2 != s0) ? m_tgt : row_max(row, false, 0);
       if (R.max_mode == 1) m = fmaxf(0.0f, m);
       m = done ? 0.0f : m;
       my_key = s0 * A + a;
@@ -359,85 +334,163 @@ __global__ __launch_bounds__(256) void k_shared_persist(const Rules R, const Ptr
         s = s2;
       }
     }
-    CRL_MARK(1);
-    // the raw samples, for an owner that finds more block sums than a cell holds
-    if (has_env) {
-      st_dev(key + env, live ? my_key : -1);
-      st_dev(delta + env, my_delta);
-    }
-
-    // 3. block sums to the owners' cells
-    reduce_block_dev(L, G, wg, my_key, my_delta, live, handoff);
     CRL_MARK(2);
-    drain_stores();
-    __syncthreads();
-    if (tid == 0) st_dev(block_flags + wg, (unsigned)(k + 1));
+
+    // ---- block sums to the owners' cells ------------------------------------------------
+    const int half = k & 1;  // cells and raw samples: two buffers, taken in turn
+    const bool over = reduce_block<true>(L.red, G, wg, my_key, my_delta, live, B.cells, want,
+                                         reinterpret_cast<unsigned long long*>(L.tile), &w_cells,
+                                         (uint32_t)((size_t)half * cells_half * 8));
+    if (over && has_env)
+      st_dev64(B.raw + (size_t)half * P.N + env, tagged(__float_as_uint(my_delta),
+                                   (uint32_t)my_key | (live ? kRawValid : 0u) | (want << kRawTagShift)));
     CRL_MARK(3);
 
-    // 4. as owner of 64 keys: all blocks' cells, added in tree order
+    // ---- while the cells travel: the owner's tile cleared, the next step prepared ----
     if (is_owner) {
-      if (!wait_flags(block_flags, n_groups, (unsigned)(k + 1), err, &lds_dead, spin_limit)) break;
-      CRL_MARK(4);
-      // (the wait's barrier also ends every thread's use of the block's LDS table)
-      const int b = tid;
-      uint4 c0 = make_uint4(0, 0, 0, 0), c1 = c0, c2 = c0, c3 = c0;
-      if (b < G.n_blocks) {
-        const uint4* src = reinterpret_cast<const uint4*>(handoff + ((size_t)wg * G.n_blocks + b) * kHandoffRecs);
-        ld_dev4x4(src, src + 1, src + 2, src + 3, c0, c1, c2, c3);
-      }
-      float4* my_row = reinterpret_cast<float4*>(tile + tid * kOwnKeys);
+      float4* tile4 = reinterpret_cast<float4*>(L.tile);
 #pragma unroll
-      for (int i = 0; i < kOwnKeys / 4; ++i) my_row[i] = make_float4(0.0f, 0.0f, 0.0f, 0.0f);
-      const int c = (int)((c0.x >> 8) & 0xFFu);
-      float* row = tile + tid * kOwnKeys;
-      if (c != kSlotOverflow) {
-        const uint4 cell[4] = {c0, c1, c2, c3};
+      for (int i = 0; i < kTileBlocks * kOwnKeys / 4 / 256; ++i) tile4[i * 256 + tid] = make_float4(0.0f, 0.0f, 0.0f, 0.0f);
+    }
+    // the cells are acknowledged before the first look at the others': asking while
+    // stores are still on their way takes longer than waiting for them (measured)
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    CRL_MARK(4);
+
+    // ---- as owner of 64 keys: all blocks' cells, added in tree order --------------------
+    if (is_owner) {
+      // A wave takes 64 blocks' cells: 4 KB that it reads side by side, 16 bytes = two
+      // records to a lane and load, so that a load of the wave is a handful of whole
+      // lines instead of 64 pieces of 64 different lines.  Lanes 4c .. 4c+3 of load j hold
+      // the eight records of block 64 * wave + 16 * j + c.
+      uint4 rec[4];
+      int cnt[4];
+      {
+        const int pair = lane & 3;
+        uint32_t src[4];  // byte offsets into the cells
+        bool have[4];
 #pragma unroll
-        for (int i = 0; i < kHandoffRecs / 2; ++i) {
-          if (c > 2 * i) row[cell[i].x & 0xFFu] = __uint_as_float(cell[i].y);
-          if (c > 2 * i + 1) row[cell[i].z & 0xFFu] = __uint_as_float(cell[i].w);
+        for (int j = 0; j < 4; ++j) {
+          const int blk = wave * 64 + j * 16 + (lane >> 2);
+          have[j] = blk < G.n_blocks;
+          src[j] = (uint32_t)(((size_t)half * cells_half + (size_t)((have[j] ? blk : 0) * n_own + wg) * kHandoffRecs + 2 * pair) * 8);
         }
-      } else {
-        // more distinct keys than slots: redo the block's part from its samples, in order
-        const int lo = b * kBlockSamples, hi = min(P.N, lo + kBlockSamples);
-        for (int i = lo; i < hi; ++i) {
-          const int kk = (int)ld_dev(reinterpret_cast<const unsigned*>(key + i));
-          if (kk >= 0 && owner_of(kk, G.own_shift) == wg) {
-            float& acc = row[kk >> G.own_shift];
-            acc = acc + __uint_as_float(ld_dev(reinterpret_cast<const unsigned*>(delta + i)));
+        bool ok = false;
+        int spins = 0;
+        for (;;) {
+          poll_fence();
+#pragma unroll
+          for (int j = 0; j < 4; ++j) rec[j] = ld_dev128(w_cells, src[j]);
+          ok = true;
+#pragma unroll
+          for (int j = 0; j < 4; ++j) {
+            const uint32_t meta0 = (uint32_t)__shfl((int)rec[j].x, lane & ~3);
+            const int c = rec_count(meta0);
+            cnt[j] = c;
+            // (every record of a cell is written every step)
+            const bool mine = rec_tag(meta0) == want && rec_tag(rec[j].x) == want && rec_tag(rec[j].z) == want;
+            ok = ok && (mine || !have[j]);
+          }
+          if (__all(ok)) break;
+          if (++spins >= spin_limit || ((spins & 63) == 0 && ld_dev32(B.err) != 0u)) {
+            L.dead = 1;
+            break;
+          }
+        }
+        if (CLK) phase_[9] += (unsigned long long)spins + 1ull;
+        __syncthreads();  // (also: the tile is clear for everybody)
+        if (L.dead) {
+          gave_up = true;
+          break;
+        }
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+          const int blk = wave * 64 + j * 16 + (lane >> 2);
+          if (have[j]) {
+            float* row = L.tile + blk * kOwnKeys;
+            if (cnt[j] == kSlotOverflow) {
+              if (pair == 0) L.o_list[atomicAdd(&L.o_count, 1)] = (uint8_t)blk;
+            } else {
+              if (2 * pair < cnt[j]) row[rec_slot(rec[j].x)] = __uint_as_float(rec[j].y);
+              if (2 * pair + 1 < cnt[j]) row[rec_slot(rec[j].z)] = __uint_as_float(rec[j].w);
+            }
           }
         }
       }
-      __syncthreads();
       CRL_MARK(5);
+      __syncthreads();
+      // blocks with more distinct keys for this owner than a cell holds: their raw
+      // samples, all threads at once, then one thread per key adds its matches in order
+      const int n_over = L.o_count;
+      bool raw_failed = false;
+      for (int q = 0; q < n_over; ++q) {
+        const int bb = L.o_list[q];
+        const int i = bb * kBlockSamples + tid;
+        int slot = 255;
+        float dv = 0.0f;
+        if (i < P.N) {
+          unsigned long long v = 0ull;
+          int spins = 0;
+          for (;;) {
+            poll_fence();
+            v = ld_dev64(B.raw + (size_t)half * P.N + i);
+            if ((tag_of(v) >> kRawTagShift) == want) break;
+            if (++spins >= spin_limit || ((spins & 63) == 0 && ld_dev32(B.err) != 0u)) {
+              raw_failed = true;
+              break;
+            }
+          }
+          const int kk = (int)(tag_of(v) & kRawKeyMask);
+          if (!raw_failed && (tag_of(v) & kRawValid) && owner_of(kk, G) == wg) {
+            slot = slot_of(kk, G);
+            dv = value_of(v);
+          }
+        }
+        L.o_slot[tid] = (uint8_t)slot;
+        L.o_delta[tid] = dv;
+        __syncthreads();
+        if (tid < kOwnKeys) {
+          float acc = 0.0f;
+          for (int j = 0; j < kBlockSamples; ++j)
+            if (L.o_slot[j] == tid) acc = acc + L.o_delta[j];  // sample order
+          L.tile[bb * kOwnKeys + tid] = acc;
+        }
+        __syncthreads();
+      }
+      if (n_over > 0) {
+        if (tid == 0) L.o_count = 0;
+        if (raw_failed) L.dead = 1;
+        __syncthreads();
+        if (L.dead) {
+          gave_up = true;
+          break;
+        }
+      }
 #pragma unroll
       for (int gi = 0; gi < 4; ++gi) {
         const int grp = wave * 4 + gi;
         float acc = 0.0f;
 #pragma unroll
-        for (int bb = 0; bb < kGroupBlocks; ++bb) acc = acc + tile[(grp * kGroupBlocks + bb) * kOwnKeys + lane];
-        gsum[grp * kOwnKeys + lane] = acc;
+        for (int bb = 0; bb < kGroupBlocks; ++bb) acc = acc + L.tile[(grp * kGroupBlocks + bb) * kOwnKeys + lane];
+        L.gsum[grp * kOwnKeys + lane] = acc;
       }
       __syncthreads();
       if (wave == 0) {
         float total = 0.0f;
 #pragma unroll
-        for (int grp = 0; grp < kTileBlocks / kGroupBlocks; ++grp) total = total + gsum[grp * kOwnKeys + lane];
-        if (own_live) {
-          q_own = q_own + total;
-          st_dev(P.Q + own_key, q_own);
-        }
-        drain_stores();
-        if (lane == 0) st_dev(owner_flags + wg, (unsigned)(k + 1));
+        for (int grp = 0; grp < kTileBlocks / kGroupBlocks; ++grp) total = total + L.gsum[grp * kOwnKeys + lane];
+        q_own = q_own + total;
+        publish(want + 1u);
       }
-      __syncthreads();  // the tile is free again before the next step clears the block's table
       CRL_MARK(6);
     }
   }
-  if (tid == 0 && (wg == 0 || wg == n_groups - 1))
-    for (int i = 0; i < 8; ++i) reinterpret_cast<unsigned long long*>(err + 8)[(wg ? 8 : 0) + i] = phase_[i];
 #undef CRL_MARK
+  if (gave_up && tid == 0) st_dev32(B.err, 1u);
+  if (CLK && B.clocks && tid == 0 && (wg == 0 || wg == (int)gridDim.x - 1))
+    for (int i = 0; i < 10; ++i) B.clocks[(wg ? 10 : 0) + i] = phase_[i];
 
+  if (own_live) P.Q[own_key] = q_own;
   if (has_env) {
     P.s[env] = s;
     P.ep_step[env] = ep_step;
@@ -450,12 +503,12 @@ __global__ __launch_bounds__(256) void k_shared_persist(const Rules R, const Ptr
 }
 
 // ---------------------------------------------------------------------------
-// Measurement helper: what a barrier over all resident workgroups costs when it is
+// Diagnostics: what a barrier over all resident workgroups costs when it is
 // built from device-scope loads and stores, in three layouts.  `mem` is zeroed
 // before the launch; out[0] receives the 100 MHz clock ticks of `rounds` barriers,
 // out[1] the number of workgroups that gave up waiting.
 //   0  one packed flag word per workgroup, every workgroup polls all of them with one
-//      16-byte load per lane (what k_shared_persist does)
+//      16-byte load per lane
 //   1  one flag per 128-byte line, polled one load at a time
 //   2  a tree in which every word has one writer and one reader: 16 members -> their
 //      leader -> the root, which releases all workgroups through one word each
@@ -464,55 +517,46 @@ constexpr int kProbeLine = 32;  // words per 128-byte line
 template <int PATTERN>
 __global__ __launch_bounds__(256) void k_probe_barrier(unsigned* mem, const int rounds, unsigned long long* out) {
   const int n = (int)gridDim.x, w = (int)blockIdx.x, tid = (int)threadIdx.x;
-  __shared__ int dead;
-  if (tid == 0) dead = 0;
-  __syncthreads();
-  auto wait_word = [&](const unsigned* p, unsigned want) {
+  constexpr int kLimit = kPersistSpinLimit / 8;
+  bool dead = false;  // the same in every thread of the workgroup
+  // -> false when the limit was hit
+  auto wait_word = [&](const unsigned* p, unsigned want) -> bool {
     int spins = 0;
-    while ((int)(ld_dev(p) - want) < 0 && ++spins < kPersistSpinLimit / 8) {}
-    if (spins >= kPersistSpinLimit / 8) dead = 1;
+    while ((int)(ld_dev32(p) - want) < 0)
+      if (++spins >= kLimit) return false;
+    return true;
   };
   const unsigned long long t0 = wall_clock64();
   for (int r = 1; r <= rounds && !dead; ++r) {
+    bool ok = true;
     if (PATTERN == 0) {
-      if (tid == 0) st_dev(mem + w, (unsigned)r);
-      if (tid < 64 && tid * 4 < n) {
-        int spins = 0;
-        for (;;) {
-          const uint4 v = ld_dev4(reinterpret_cast<const uint4*>(mem + tid * 4));
-          const bool ok = (int)(v.x - r) >= 0 && (tid * 4 + 1 >= n || (int)(v.y - r) >= 0) &&
-                          (tid * 4 + 2 >= n || (int)(v.z - r) >= 0) && (tid * 4 + 3 >= n || (int)(v.w - r) >= 0);
-          if (ok) break;
-          if (++spins >= kPersistSpinLimit / 8) {
-            dead = 1;
-            break;
-          }
-        }
-      }
-    } else if (PATTERN == 1) {
-      if (tid == 0) st_dev(mem + (size_t)w * kProbeLine, (unsigned)r);
+      if (tid == 0) st_dev32(mem + w, (unsigned)r);
       if (tid < 64)
-        for (int i = tid; i < n; i += 64) wait_word(mem + (size_t)i * kProbeLine, (unsigned)r);
+        for (int i = tid * 4; i < min(n, tid * 4 + 4); ++i) ok = ok && wait_word(mem + i, (unsigned)r);
+    } else if (PATTERN == 1) {
+      if (tid == 0) st_dev32(mem + (size_t)w * kProbeLine, (unsigned)r);
+      if (tid < 64)
+        for (int i = tid; i < n; i += 64) ok = ok && wait_word(mem + (size_t)i * kProbeLine, (unsigned)r);
     } else {
       unsigned* arrive = mem;                        // [16 groups][line]: word m of group g
       unsigned* garrive = mem + 16 * kProbeLine;     // word g
       unsigned* go = mem + 17 * kProbeLine;          // [workgroup][line]
       const int g = w >> 4, m = w & 15;
       const int members = min(16, n - g * 16), groups = (n + 15) >> 4;
-      if (tid == 0) st_dev(arrive + g * kProbeLine + m, (unsigned)r);
+      if (tid == 0) st_dev32(arrive + g * kProbeLine + m, (unsigned)r);
       if (m == 0) {
-        if (tid < members) wait_word(arrive + g * kProbeLine + tid, (unsigned)r);
-        __syncthreads();
-        if (tid == 0) st_dev(garrive + g, (unsigned)r);
+        if (tid < members) ok = wait_word(arrive + g * kProbeLine + tid, (unsigned)r);
+        ok = __syncthreads_or(!ok) == 0;
+        if (tid == 0) st_dev32(garrive + g, (unsigned)r);
         if (w == 0) {
-          if (tid < groups) wait_word(garrive + tid, (unsigned)r);
-          __syncthreads();
-          if (tid < n) st_dev(go + (size_t)tid * kProbeLine, (unsigned)r);
+          if (tid < groups) ok = ok && wait_word(garrive + tid, (unsigned)r);
+          ok = __syncthreads_or(!ok) == 0;
+          if (tid < n) st_dev32(go + (size_t)tid * kProbeLine, (unsigned)r);
         }
       }
-      if (tid == 0) wait_word(go + (size_t)w * kProbeLine, (unsigned)r);
+      if (tid == 0) ok = ok && wait_word(go + (size_t)w * kProbeLine, (unsigned)r);
     }
-    __syncthreads();
+    dead = __syncthreads_or(!ok) != 0;  // every thread leaves the loop in the same round
   }
   if (tid == 0 && dead) atomicAdd(out + 1, 1ull);
   if (tid == 0 && w == 0) out[0] = wall_clock64() - t0;

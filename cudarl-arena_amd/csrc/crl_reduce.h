@@ -7,10 +7,11 @@
 //   total  = group sums added left to right from +0.0f;   Q[k] = Q[k] + total[k]
 //
 // Two passes over the chip:
-//   1. one workgroup per block walks its 256 samples in order (wave after wave;
-//      inside a wave the lanes that share a key are found with ballots and
-//      folded in lane order) keeping the running sums in a dense LDS table, and
-//      hands every distinct key's block sum to the workgroup that owns the key;
+//   1. one workgroup per block: the lowest thread that holds a key becomes the
+//      key's leader (LDS atomic min on a dense table), the other holders mark
+//      themselves in the leader's 256-bit member set (LDS atomic or), and the
+//      leader adds the members' deltas in thread order = sample order; every
+//      distinct key's block sum goes to the workgroup that owns the key;
 //   2. one workgroup per 64 keys lays the block sums it was handed out as a
 //      dense [block][key] tile in LDS and adds the columns in the tree order.
 // Empty blocks add +0.0f, which changes nothing, so the result is a pure
@@ -23,125 +24,220 @@ namespace crl {
 
 constexpr int kBlockSamples = 256;   // level 0
 constexpr int kGroupBlocks = 16;     // level 1
-constexpr int kOwnKeys = 64;         // keys per owner workgroup
+constexpr int kOwnKeys = 64;         // keys per owner workgroup: 64 / A whole table rows
 constexpr int kSlotCap = 8;          // block sums one block can hand one owner
-constexpr int kHandoffRecs = 8;      // one 64-byte hand-off cell of 8 records {key slot | count << 8, sum}
-constexpr int kSlotOverflow = 255;   // count value: read the block's raw samples instead
+constexpr int kHandoffRecs = 8;      // one 64-byte hand-off cell of 8 records
+constexpr int kSlotOverflow = 15;    // count value: read the block's raw samples instead
 constexpr int kDenseKeys = 16384;    // keys the dense LDS table of pass 1 can hold
 constexpr int kTileBlocks = 256;     // blocks per LDS tile of pass 2
-constexpr uint32_t kOwnerMix = 37;   // odd: spreads neighbouring keys over owners
+constexpr uint32_t kOwnerMix = 37;   // odd: spreads cells a power of two apart over owners
+constexpr uint32_t kNoLead = 0xFFFFFFFFu;
+
+// A hand-off record is 64 bits, written and read as one unit:
+//   bits  0..5   slot of the key among its owner's 64
+//   bits  6..9   record 0 of a cell only: how many records the cell holds
+//                (0: none, kSlotOverflow: more than kSlotCap distinct keys)
+//   bits 10..31  step tag (the one-launch kernel: a record is valid once its tag is
+//                the step's; 0 where launches separate the steps)
+//   bits 32..63  the block sum, fp32
+constexpr int kRecCountShift = 6, kRecTagShift = 10;
+constexpr uint32_t kRecTagMask = (1u << (32 - kRecTagShift)) - 1u;
+__device__ __forceinline__ unsigned long long make_rec(uint32_t slot, uint32_t count, uint32_t tag, float v) {
+  const uint32_t meta = slot | (count << kRecCountShift) | (tag << kRecTagShift);
+  return (unsigned long long)meta | ((unsigned long long)__float_as_uint(v) << 32);
+}
+__device__ __forceinline__ int rec_slot(uint32_t meta) { return (int)(meta & 63u); }
+__device__ __forceinline__ int rec_count(uint32_t meta) { return (int)((meta >> kRecCountShift) & 15u); }
+__device__ __forceinline__ uint32_t rec_tag(uint32_t meta) { return meta >> kRecTagShift; }
 
 struct ReduceGeom {
-  int K;          // keys of the table
-  int key_bits;   // ceil(log2 K)
+  int K;          // keys of the table, key = cell * A + action
+  int a_shift;    // log2(A)
   int own_shift;  // log2(number of owners); owners = 1 << own_shift, (K >> own_shift) <= 64
   int n_blocks;   // ceil(n / 256)
 };
 
-// key <-> (owner, slot in the owner's 64): slot = key >> own_shift,
-// owner = (low bits + 37 * slot) mod owners
-__device__ __forceinline__ int owner_of(int key, int own_shift) {
-  const uint32_t mask = (1u << own_shift) - 1u;
-  const uint32_t hi = (uint32_t)key >> own_shift;
-  return (int)(((uint32_t)key + kOwnerMix * hi) & mask);
+// key <-> (owner, slot in the owner's 64).  An owner holds whole table rows:
+// hi = cell >> own_shift, owner = (cell + 37 * hi) mod owners, slot = hi * A + action
+__device__ __forceinline__ int owner_of(int key, const ReduceGeom& G) {
+  const uint32_t mask = (1u << G.own_shift) - 1u;
+  const uint32_t cell = (uint32_t)key >> G.a_shift;
+  return (int)((cell + kOwnerMix * (cell >> G.own_shift)) & mask);
 }
-__device__ __forceinline__ int key_of(int owner, int slot, int own_shift) {
-  const uint32_t mask = (1u << own_shift) - 1u;
-  const uint32_t lo = ((uint32_t)owner - kOwnerMix * (uint32_t)slot) & mask;
-  return (int)(((uint32_t)slot << own_shift) | lo);
+__device__ __forceinline__ int slot_of(int key, const ReduceGeom& G) {
+  const uint32_t cell = (uint32_t)key >> G.a_shift;
+  return (int)(((cell >> G.own_shift) << G.a_shift) | ((uint32_t)key & ((1u << G.a_shift) - 1u)));
+}
+__device__ __forceinline__ int key_of(int owner, int slot, const ReduceGeom& G) {
+  const uint32_t mask = (1u << G.own_shift) - 1u;
+  const uint32_t hi = (uint32_t)slot >> G.a_shift;
+  const uint32_t lo = ((uint32_t)owner - kOwnerMix * hi) & mask;
+  const uint32_t cell = (hi << G.own_shift) | lo;
+  return (int)((cell << G.a_shift) | ((uint32_t)slot & ((1u << G.a_shift) - 1u)));
 }
 
-struct ReduceLds {
-  float run[kDenseKeys];      // running sum of the block, per key
-  uint8_t seen[kDenseKeys];   // key touched by this block
-  int handed[256];            // block sums handed to each owner so far
+// ---- device-scope accesses --------------------------------------------------------
+// gfx950 has eight XCDs, each with its own L2; plain loads and stores are coherent
+// inside one XCD only.  Relaxed atomic loads and stores at agent scope compile to
+// accesses that carry the sc1 bit and are served past the L2: a value stored that
+// way by one workgroup is seen by the next such load of any other, without the
+// whole-L2 write-back / invalidate of a release / acquire fence.  64 bits is the
+// unit: every exchanged datum carries its own step tag in the same 64 bits, so no
+// ordering between two stores is ever relied on.
+__device__ __forceinline__ void st_dev64(unsigned long long* p, unsigned long long v) {
+  __hip_atomic_store(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+__device__ __forceinline__ unsigned long long ld_dev64(const unsigned long long* p) {
+  return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+__device__ __forceinline__ void st_dev32(unsigned* p, unsigned v) {
+  __hip_atomic_store(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+__device__ __forceinline__ unsigned ld_dev32(const unsigned* p) {
+  return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+// Aligned 16-byte device-scope loads: a buffer load with the sc1 bit, through a window
+// (buffer descriptor) that starts at `base` and spans 2 GB.  Each aligned 64-bit half is
+// one of the tagged units above; nothing is assumed about the two halves of a load
+// belonging together.  To the compiler this is an ordinary read of memory: a loop that
+// asks again and again must call poll_fence() in every round, or the load is taken out
+// of the loop as invariant.
+typedef unsigned int crl_u4 __attribute__((ext_vector_type(4)));
+using DevWindow = __amdgpu_buffer_rsrc_t;
+__device__ __forceinline__ DevWindow dev_window(const void* base) {
+  return __builtin_amdgcn_make_buffer_rsrc(const_cast<void*>(base), 0, 0x7fffffff, 0x00020000);
+}
+__device__ __forceinline__ uint4 ld_dev128(DevWindow w, uint32_t byte_offset) {
+  const crl_u4 v = __builtin_amdgcn_raw_buffer_load_b128(w, (int)byte_offset, 0, 16 /* sc1 */);
+  return make_uint4(v.x, v.y, v.z, v.w);
+}
+__device__ __forceinline__ void st_dev128(DevWindow w, uint32_t byte_offset, const uint4 v) {
+  crl_u4 t;
+  t.x = v.x;
+  t.y = v.y;
+  t.z = v.z;
+  t.w = v.w;
+  __builtin_amdgcn_raw_buffer_store_b128(t, w, (int)byte_offset, 0, 16 /* sc1 */);
+}
+__device__ __forceinline__ void poll_fence() { asm volatile("" ::: "memory"); }
+
+struct alignas(16) ReduceLds {  // (lead and members are also accessed 16 bytes at a time)
+  alignas(16) uint32_t lead[kDenseKeys];                     // lowest thread of the block that holds the key; kNoLead between uses
+  alignas(16) unsigned long long members[kBlockSamples][4];  // per leader: the threads that hold its key; zero between uses
+  float delta[kBlockSamples];
+  int handed[256];                               // block sums handed to each owner
+  int over;                                      // some owner was handed more than a cell holds
 };
 
-// Clears the block's LDS state.  Needs no sample, so a kernel calls it first and
-// lets it overlap with the loads that produce the samples; reduce_block() has the
-// barrier that orders it before the first use.
-__device__ __forceinline__ void reduce_block_clear(ReduceLds& L, const ReduceGeom G) {
+// Once per kernel, before the first reduce_block() and separated from it by a barrier.
+__device__ __forceinline__ void reduce_block_init(ReduceLds& L) {
   const int tid = threadIdx.x;
-  uint4* seen4 = reinterpret_cast<uint4*>(L.seen);
-  for (int i = tid; i < kDenseKeys / 16; i += kBlockSamples) seen4[i] = make_uint4(0, 0, 0, 0);
-  if (tid < (1 << G.own_shift)) L.handed[tid] = 0;
+  uint4* lead4 = reinterpret_cast<uint4*>(L.lead);
+  for (int i = tid; i < kDenseKeys / 4; i += kBlockSamples) lead4[i] = make_uint4(kNoLead, kNoLead, kNoLead, kNoLead);
+  L.members[tid][0] = 0ull;
+  L.members[tid][1] = 0ull;
+  L.members[tid][2] = 0ull;
+  L.members[tid][3] = 0ull;
+  if (tid == 0) L.over = 0;
 }
 
-// Pass 1 for one block, after reduce_block_clear().  All 256 threads of the
-// workgroup call it with their sample (valid = false: no sample / no delta).
-// key < K <= kDenseKeys.
-__device__ __forceinline__ void reduce_block(ReduceLds& L, const ReduceGeom G, const int block,
-                                             const int key, const float delta, const bool valid,
-                                             uint2* __restrict__ handoff) {
-  const int tid = threadIdx.x;
-  const int lane = tid & 63;
-  const int wave = tid >> 6;
-  const int n_own = 1 << G.own_shift;
+// Pass 1 for one block.  All 256 threads of the workgroup call it with their
+// sample (valid = false: no sample / no delta); key < K <= kDenseKeys.  Leaves the
+// LDS state as reduce_block_init() did, so it can be called again and again.
+// The hand-off cell of (block, owner) is 64 bytes at handoff[(block * owners + owner) * 8].
+// DEV = false: the records go straight to memory with plain stores, for a reader in a
+// later launch.
+// DEV = true: for readers on other XCDs in the same launch.  All cells of the block
+// are put together in LDS (`stage`, owners x 8 records, free again on return) and go
+// out as whole lines, 16 bytes to a store and lane, every record carrying `tag`:
+// scattered 8-byte stores are partial line writes, and some 350 of them per workgroup
+// took 1.6 us to be acknowledged.  `window` is a buffer window on `handoff`.
+// Returns (to every thread) whether some owner was handed more than kSlotCap
+// distinct keys: its cell then says kSlotOverflow and the owner needs the block's
+// raw samples.
+// DEV = true: before each reduce_block(), separated from it by a barrier (and from the
+// one before by another): every record of every cell starts as "nothing, of this step".
+// Thread t touches the 16-byte pieces t, t + 256, ... of `stage` here and on the way out
+// of reduce_block(), and no others.
+__device__ __forceinline__ void reduce_stage_init(unsigned long long* stage, const ReduceGeom G, const uint32_t tag) {
+  const unsigned long long none = make_rec(0u, 0u, tag, 0.0f);
+  ulonglong2* stage2 = reinterpret_cast<ulonglong2*>(stage);
+  for (int i = threadIdx.x; i < (kHandoffRecs / 2) << G.own_shift; i += kBlockSamples) stage2[i] = make_ulonglong2(none, none);
+}
 
-  // lanes of this wave that hold the same key
-  unsigned long long peers = __ballot(valid);
-  for (int b = 0; b < G.key_bits; ++b) {
-    const bool bit = (key >> b) & 1;
-    const unsigned long long m = __ballot(bit);
-    peers &= bit ? m : ~m;
-  }
-  const bool leader = valid && (peers & ((1ull << lane) - 1ull)) == 0ull;
-  const int owner = owner_of(key, G.own_shift);
-  bool first = false;
-  int slot = 0;
-  // The waves take turns below (a key's running sum passes from wave to wave), so
-  // what can be done before a wave's turn is done here, by all waves at once: a
-  // leader fetches the deltas of its first eight samples, itself included.  Absent
-  // ones are +0.0f, which leaves a sum that started from +0.0f unchanged.
-  constexpr int kAhead = 8;
-  unsigned long long rest = leader ? peers : 0ull;
-  float ahead[kAhead];
-#pragma unroll
-  for (int i = 0; i < kAhead; ++i) {
-    const int j = rest ? __builtin_ctzll(rest) : lane;
-    const float dj = __shfl(delta, j);
-    ahead[i] = rest ? dj : 0.0f;
-    rest &= rest - 1ull;
+template <bool DEV>
+__device__ __forceinline__ bool reduce_block(ReduceLds& L, const ReduceGeom G, const int block,
+                                             const int key, const float delta, const bool valid,
+                                             unsigned long long* handoff, const uint32_t tag,
+                                             unsigned long long* stage = nullptr, const DevWindow* window = nullptr,
+                                             const uint32_t window_offset = 0) {
+  const int tid = threadIdx.x;
+  const int n_own = 1 << G.own_shift;
+  if (valid) atomicMin(&L.lead[key], (uint32_t)tid);
+  L.delta[tid] = delta;
+  __syncthreads();
+  L.handed[tid] = 0;  // (256 >= owners; the last call's readers are past the barrier above)
+  if (tid == 0) L.over = 0;
+  uint32_t ld = (uint32_t)tid;
+  if (valid) {
+    ld = L.lead[key];
+    if (ld != (uint32_t)tid) atomicOr(&L.members[ld][tid >> 6], 1ull << (tid & 63));
   }
   __syncthreads();
-
-  for (int w = 0; w < 4; ++w) {
-    if (wave == w) {
-      float acc = 0.0f;
-      if (leader) {
-        first = L.seen[key] == 0;
-        acc = first ? 0.0f : L.run[key];
-      }
+  const bool leader = valid && ld == (uint32_t)tid;
+  float acc = 0.0f;
+  int slot = 0, owner = 0;
+  if (leader) {
+    acc = acc + delta;  // the leader is the key's first sample; the other holders come after it
+    const ulonglong2 lo = *reinterpret_cast<const ulonglong2*>(&L.members[tid][0]);
+    const ulonglong2 hi = *reinterpret_cast<const ulonglong2*>(&L.members[tid][2]);
+    unsigned long long mw[4] = {lo.x, lo.y, hi.x, hi.y};
+    if ((mw[0] | mw[1] | mw[2] | mw[3]) != 0ull) {
+      *reinterpret_cast<ulonglong2*>(&L.members[tid][0]) = make_ulonglong2(0ull, 0ull);
+      *reinterpret_cast<ulonglong2*>(&L.members[tid][2]) = make_ulonglong2(0ull, 0ull);
 #pragma unroll
-      for (int i = 0; i < kAhead; ++i) acc = acc + ahead[i];  // lane order = sample order
-      while (__ballot(rest != 0ull) != 0ull) {  // the rare key with more than eight samples in a wave
-        const int j = rest ? __builtin_ctzll(rest) : lane;
-        const float dj = __shfl(delta, j);
-        if (rest) acc = acc + dj;  // lane order = sample order
-        rest &= rest - 1ull;
-      }
-      if (leader) {
-        L.run[key] = acc;
-        L.seen[key] = 1;
-        if (first) slot = atomicAdd(&L.handed[owner], 1);  // slot order is free: records carry the key
+      for (int w = 0; w < 4; ++w) {
+        unsigned long long m = mw[w];
+        while (m != 0ull) {
+          const int j = __builtin_ctzll(m);
+          acc = acc + L.delta[w * 64 + j];  // thread order = sample order
+          m &= m - 1ull;
+        }
       }
     }
-    __syncthreads();
+    L.lead[key] = kNoLead;
+    owner = owner_of(key, G);
+    slot = atomicAdd(&L.handed[owner], 1);  // slot order is free: records carry the key
+    if (slot >= kSlotCap) L.over = 1;
+    // (record 0's count is added on the way out, when every leader has drawn its slot)
+    if (DEV && slot < kSlotCap) stage[owner * kHandoffRecs + slot] = make_rec((uint32_t)slot_of(key, G), 0u, tag, acc);
   }
+  __syncthreads();
+  const bool over = L.over != 0;
 
-  // hand-off cell of (owner, block): 64 bytes that the owner gets with one
-  // independent read; record 0 also carries the count (0: nothing for this owner)
-  if (leader && first && slot < kSlotCap) {
-    const size_t at = ((size_t)owner * G.n_blocks + block) * kHandoffRecs + slot;
-    uint32_t tag = (uint32_t)(key >> G.own_shift);
-    if (slot == 0) {
-      const int c = L.handed[owner];  // final: every wave has had its turn
-      tag |= (uint32_t)(c > kSlotCap ? kSlotOverflow : c) << 8;
+  if (DEV) {
+    const ulonglong2* stage2 = reinterpret_cast<const ulonglong2*>(stage);
+    for (int i = tid; i < n_own * (kHandoffRecs / 2); i += kBlockSamples) {
+      ulonglong2 v = stage2[i];
+      if ((i & 3) == 0) {
+        const int c = L.handed[i >> 2];
+        v.x |= (unsigned long long)(uint32_t)(c > kSlotCap ? kSlotOverflow : c) << kRecCountShift;
+      }
+      st_dev128(*window, window_offset + (uint32_t)(((size_t)block * n_own * kHandoffRecs + (size_t)i * 2) * 8),
+                make_uint4((uint32_t)v.x, (uint32_t)(v.x >> 32), (uint32_t)v.y, (uint32_t)(v.y >> 32)));
     }
-    handoff[at] = make_uint2(tag, __float_as_uint(L.run[key]));
+  } else {
+    if (leader && slot < kSlotCap) {
+      uint32_t count = 0;
+      if (slot == 0) {
+        const int c = L.handed[owner];  // final: every leader has drawn its slot
+        count = (uint32_t)(c > kSlotCap ? kSlotOverflow : c);
+      }
+      handoff[((size_t)block * n_own + owner) * kHandoffRecs + slot] = make_rec((uint32_t)slot_of(key, G), count, tag, acc);
+    }
+    if (tid < n_own && L.handed[tid] == 0) handoff[((size_t)block * n_own + tid) * kHandoffRecs] = make_rec(0u, 0u, tag, 0.0f);
   }
-  if (tid < n_own && L.handed[tid] == 0)
-    handoff[((size_t)tid * G.n_blocks + block) * kHandoffRecs] = make_uint2(0u, 0u);
+  return over;
 }
 
 // Pass 1 over (key, delta) arrays already in memory.
@@ -149,23 +245,24 @@ __global__ __launch_bounds__(kBlockSamples) void k_reduce_blocks(const ReduceGeo
                                                                  const int32_t* __restrict__ key,
                                                                  const float* __restrict__ delta,
                                                                  const int n,
-                                                                 uint2* __restrict__ handoff) {
-  extern __shared__ unsigned char lds_raw[];
+                                                                 unsigned long long* __restrict__ handoff) {
+  extern __shared__ __align__(16) unsigned char lds_raw[];
   ReduceLds& L = *reinterpret_cast<ReduceLds*>(lds_raw);
-  reduce_block_clear(L, G);
+  reduce_block_init(L);
   const int i = blockIdx.x * kBlockSamples + threadIdx.x;
   const int k = i < n ? key[i] : -1;
   const bool valid = k >= 0;
   const float d = valid ? delta[i] : 0.0f;
-  reduce_block(L, G, blockIdx.x, valid ? k : 0, d, valid, handoff);
+  __syncthreads();
+  reduce_block<false>(L, G, blockIdx.x, valid ? k : 0, d, valid, handoff, 0u);
 }
 
 // Pass 2: one workgroup per owner (64 keys).
 __global__ __launch_bounds__(256) void k_reduce_owners(const ReduceGeom G, float* __restrict__ Q,
                                                         const int32_t* __restrict__ key,
                                                         const float* __restrict__ delta, const int n,
-                                                        const uint2* __restrict__ handoff) {
-  extern __shared__ float tile[];  // [kTileBlocks][64] block sums, then [16][64] group sums
+                                                        const unsigned long long* __restrict__ handoff) {
+  extern __shared__ __align__(16) float tile[];  // [kTileBlocks][64] block sums, then [16][64] group sums
   float* gsum = tile + kTileBlocks * kOwnKeys;
   const int tid = threadIdx.x;
   const int lane = tid & 63;
@@ -173,7 +270,7 @@ __global__ __launch_bounds__(256) void k_reduce_owners(const ReduceGeom G, float
   const int owner = blockIdx.x;
   float total = 0.0f;
   // the table entry this lane will update: fetched now, needed last
-  const int my_key = key_of(owner, lane, G.own_shift);
+  const int my_key = key_of(owner, lane, G);
   const float q_old = (wave == 0 && my_key < G.K) ? Q[my_key] : 0.0f;
 
   for (int b0 = 0; b0 < G.n_blocks; b0 += kTileBlocks) {
@@ -181,31 +278,34 @@ __global__ __launch_bounds__(256) void k_reduce_owners(const ReduceGeom G, float
     // the whole hand-off cell in one go: no load depends on another
     uint4 cell[kHandoffRecs / 2];
     if (b < G.n_blocks) {
-      const uint4* src = reinterpret_cast<const uint4*>(handoff + ((size_t)owner * G.n_blocks + b) * kHandoffRecs);
+      const uint4* src = reinterpret_cast<const uint4*>(handoff + ((size_t)b * (1 << G.own_shift) + owner) * kHandoffRecs);
 #pragma unroll
       for (int i = 0; i < kHandoffRecs / 2; ++i) cell[i] = src[i];
     } else {
 #pragma unroll
       for (int i = 0; i < kHandoffRecs / 2; ++i) cell[i] = make_uint4(0, 0, 0, 0);
     }
-    float4* my_row = reinterpret_cast<float4*>(tile + tid * kOwnKeys);
+    // the tile is cleared by all threads side by side (a thread clearing its own row
+    // would put all 64 lanes of a store on the same LDS banks)
+    float4* tile4 = reinterpret_cast<float4*>(tile);
 #pragma unroll
-    for (int i = 0; i < kOwnKeys / 4; ++i) my_row[i] = make_float4(0.0f, 0.0f, 0.0f, 0.0f);
-    const int c = (int)((cell[0].x >> 8) & 0xFFu);
+    for (int i = 0; i < kTileBlocks * kOwnKeys / 4 / 256; ++i) tile4[i * 256 + tid] = make_float4(0.0f, 0.0f, 0.0f, 0.0f);
+    __syncthreads();
+    const int c = rec_count(cell[0].x);
     if (c != kSlotOverflow) {
       float* row = tile + tid * kOwnKeys;
 #pragma unroll
       for (int i = 0; i < kHandoffRecs / 2; ++i) {
-        if (c > 2 * i) row[cell[i].x & 0xFFu] = __uint_as_float(cell[i].y);
-        if (c > 2 * i + 1) row[cell[i].z & 0xFFu] = __uint_as_float(cell[i].w);
+        if (c > 2 * i) row[rec_slot(cell[i].x)] = __uint_as_float(cell[i].y);
+        if (c > 2 * i + 1) row[rec_slot(cell[i].z)] = __uint_as_float(cell[i].w);
       }
     } else {
       // more distinct keys than slots: redo the block's part from its samples, in order
       const int lo = b * kBlockSamples, hi = min(n, lo + kBlockSamples);
       for (int i = lo; i < hi; ++i) {
         const int k = key[i];
-        if (k >= 0 && owner_of(k, G.own_shift) == owner) {
-          float& acc = tile[tid * kOwnKeys + (k >> G.own_shift)];
+        if (k >= 0 && owner_of(k, G) == owner) {
+          float& acc = tile[tid * kOwnKeys + slot_of(k, G)];
           acc = acc + delta[i];
         }
       }

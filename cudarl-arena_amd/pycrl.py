@@ -71,6 +71,9 @@ def make_config(n_envs, width, height, n_actions=4, table_mode=TABLE_PER_ENV, ma
     return c
 
 
+E_ARG, E_DEVICE, E_ALLOC, E_STATE, E_RANGE = -1, -2, -3, -4, -5  # include/crl.h
+
+
 class CrlError(RuntimeError):
     def __init__(self, code, text):
         super().__init__("crl status %d: %s" % (code, text))
@@ -87,7 +90,7 @@ EXPORTS = [
     "crl_set_state", "crl_get_episode_stats", "crl_get_step_count", "crl_set_step_count", "crl_q_get", "crl_q_set",
     "crl_q_get_range", "crl_set_trace", "crl_get_trace", "crl_set_exploration_stream", "crl_set_persist_spin_limit",
     "crl_device_ptr", "crl_fused_kernel_info", "crl_fused_plan_for_config", "crl_philox4x32_10", "crl_explore_draw",
-    "crl_eps_table", "crl_gen_maps_bernoulli", "crl_gen_maps_noise", "crl_probe_copy", "crl_probe_barrier", "crl_get_persist_clocks",
+    "crl_eps_table", "crl_gen_maps_bernoulli", "crl_gen_maps_noise", "crl_probe_copy", "crl_probe_barrier", "crl_get_persist_clocks", "crl_set_persist_clocks",
 ]
 
 
@@ -147,6 +150,7 @@ def load():
     lib.crl_probe_copy.argtypes = [C.c_size_t, C.c_int]
     lib.crl_probe_barrier.argtypes = [C.c_int, C.c_int, C.c_int, C.POINTER(C.c_double)]
     lib.crl_get_persist_clocks.argtypes = [vp, vp]
+    lib.crl_set_persist_clocks.argtypes = [vp, C.c_int32]
     _lib = lib
     return lib
 
@@ -374,11 +378,16 @@ class Engine:
     def set_persist_spin_limit(self, polls):
         _check(self.lib.crl_set_persist_spin_limit(self.h, polls))
 
+    def set_persist_clocks(self, on):
+        _check(self.lib.crl_set_persist_clocks(self.h, 1 if on else 0))
+
     def persist_clocks(self):
-        """Per-phase shader clocks of the last one-launch shared-table call: (first, last workgroup) x 8."""
-        out = np.zeros(16, np.uint64)
+        """Per-phase shader clocks of the last one-launch shared-table launch that ran with the
+        clocks armed: (first, last workgroup) x 8."""
+        out = np.zeros(20 + 8 * 256, np.uint64)
         _check(self.lib.crl_get_persist_clocks(self.h, _ptr(out)))
-        return out.reshape(2, 8)
+        self.persist_stamps = out[20:].reshape(256, 8)  # 100 MHz wall clock of every workgroup at the marks of the middle step
+        return out[:20].reshape(2, 10)
 
     def fused_kernel_info(self, n_steps=0):
         """Plan of crl_run_fused(n_steps); 0 = a long launch."""

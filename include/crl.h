@@ -202,18 +202,19 @@ int crl_td_update(crl_engine* e, int32_t table, int32_t n, const int32_t* s, con
  * crl_select; crl_step(NULL); crl_update. */
 int crl_run_fused(crl_engine* e, int32_t n_steps);
 
-/* crl_run_fused for callers that cannot allocate device memory (work recorded
- * under HIP graph capture, tight serving loops, harnesses that forbid
- * hipMalloc): no counterpart in the reference.  Same results as crl_run_fused,
- * but its scratch - the ticket counters of the per-env kernels, the hand-off
- * cells of the shared table's ordered reduction, the step flags of the one-launch
- * shared-table kernel - lives in a static device
- * array of 8 MB + 4 KB that each GPU the library runs on holds until the
- * process ends, and the call allocates and frees nothing (device or host).
- * CRL_E_RANGE if the engine's reduction needs more hand-off cells than the
- * array holds (65,536 envs on a 64x64x4 table need 4 MB).  All engines on one
- * GPU share that GPU's array: calls that overlap in time on one GPU (different
- * streams or threads) race; calls in stream order do not. */
+/* crl_run_fused for callers that cannot allocate device memory (tight serving
+ * loops, harnesses that forbid hipMalloc): no counterpart in the reference.
+ * Same results as crl_run_fused, but its scratch - the ticket counters of the
+ * per-env kernels, the hand-off cells of the shared table's ordered reduction,
+ * the exchange buffers of the one-launch shared-table kernel - lives in a
+ * static device array of 10 MB + 4 KB that each GPU the library runs on holds
+ * until the process ends, and the call allocates and frees nothing (device or
+ * host).  CRL_E_RANGE if the engine's ordered reduction needs more hand-off cells
+ * than the array holds (65,536 envs on a 64x64x4 table need 4 MB with two launches
+ * per step, 9.2 MB of exchange buffers in the one-launch kernel; an engine whose
+ * one-launch buffers do not fit takes two launches per step).  All engines on one GPU share that GPU's
+ * array: calls that overlap in time on one GPU (different streams or threads)
+ * race; calls in stream order do not. */
 int crl_run_fused_noalloc(crl_engine* e, int32_t n_steps);
 
 /* Environment getters (src/environment.h:26-37) for all envs; any pointer may
@@ -256,17 +257,22 @@ int crl_get_trace(crl_engine* e, int32_t n_steps, int32_t* s_next, uint8_t* acti
 int crl_set_exploration_stream(crl_engine* e, int32_t n_steps, const float* u,
                                const int32_t* a_rand);
 
-/* How many polls a workgroup of the one-launch shared-table kernel waits for its
- * peers before it gives up (default 2^20, a few hundred milliseconds).  A workgroup
- * that gives up sets a word that the others see and leave on; the next call that
- * synchronises (crl_sync, crl_get_state, crl_q_get, crl_get_trace) then fails with
- * CRL_E_DEVICE and the engine's state and table are not valid any more.  With a
- * limit of 1 every workgroup leaves at its first unanswered poll: how the tests
- * exercise that path without a kernel that hangs. */
+/* How many polls a thread of the one-launch shared-table kernel waits for its
+ * peers' data before it gives up (default 2^20, a few hundred milliseconds).  A
+ * workgroup that gives up sets a word that the others see and leave on, and that
+ * makes later launches of the kernel return at once; the next call that
+ * synchronises (crl_sync, crl_get_state, crl_q_get, crl_get_trace,
+ * crl_get_episode_stats) fails with CRL_E_DEVICE, once.  The engine's state and
+ * table are not valid from then on: every call that works on them fails with
+ * CRL_E_STATE until the caller sets them again (crl_reset, crl_set_state or
+ * crl_q_set).  With a limit of 1 every workgroup leaves at its first unanswered
+ * poll: how the tests exercise that path without a kernel that hangs. */
 int crl_set_persist_spin_limit(crl_engine* e, int32_t polls);
 
 /* raw device pointers of the SoA state for zero-copy consumers; index with
- * CRL_PTR_*.  Valid until crl_destroy. */
+ * CRL_PTR_*.  Valid until crl_destroy.  What they point at is the engine's as
+ * of the last call on its stream: call crl_sync first (which also reports a
+ * one-launch kernel that gave up). */
 enum {
   CRL_PTR_S = 0, CRL_PTR_EP_STEP = 1, CRL_PTR_EPISODE = 2, CRL_PTR_REWARD = 3,
   CRL_PTR_DONE = 4, CRL_PTR_ACTION = 5, CRL_PTR_Q = 6, CRL_PTR_COUNT = 7
@@ -286,21 +292,26 @@ int crl_fused_kernel_info(crl_engine* e, int32_t n_steps, char* name, size_t nam
 int crl_fused_plan_for_config(const crl_config* cfg, int32_t n_steps, char* name, size_t name_len,
                               int32_t* grid, int32_t* block, int32_t* lds_bytes);
 
-/* Measurement helper (no reference counterpart): one launch of a plain copy
- * kernel `k_probe_copy` moving n_bytes from one device buffer to another, so
- * that hardware traffic counters can be scaled by a launch of known size. */
+/* -- diagnostics (no reference counterpart; not part of the drop-in surface) -- */
+
+/* One launch of a plain copy kernel `k_probe_copy` moving n_bytes from one device
+ * buffer to another, so that hardware traffic counters can be scaled by a launch
+ * of known size. */
 int crl_probe_copy(size_t n_bytes, int repeats);
 
-/* Tuning aid (no reference counterpart): per-phase shader clocks, summed over the
- * steps of the last one-launch shared-table call (crl_set_fused_variant 2), of its
- * first (out16[0..7]) and last (out16[8..15]) workgroup.  Phases: wait for the
- * owners' table, act, block sums, drain + publish, wait for the blocks' cells,
- * cells into the tile, tile sums + publish, loop overhead. */
+/* Phase clocks of the one-launch shared-table kernel.  crl_set_persist_clocks(e, 1)
+ * makes later launches run the instantiation that reads the shader clock between
+ * the phases of every step (off by default: the product kernel carries no clocks);
+ * crl_get_persist_clocks returns the sums over the steps of the last such launch for
+ * its first (out16[0..7]) and last (out16[8..15]) workgroup.  Phases: 0 work that
+ * does not need the table, 1 wait for the table, 2 select / move / delta, 3 ordered
+ * block sums + cells, 4 clearing the owner's tile, 5 wait for the cells, 6 tile,
+ * sums, publish, 7 loop overhead. */
+int crl_set_persist_clocks(crl_engine* e, int32_t on);
 int crl_get_persist_clocks(crl_engine* e, uint64_t* out16);
-/* Measurement helper (no reference counterpart): nanoseconds per barrier over
- * n_groups (<= 256) co-resident workgroups that meet through device-scope loads
- * and stores.  pattern 0: packed flags, all polled by everybody with 16-byte
- * loads; 1: one flag per 128-byte line; 2: a tree in which every word has one
+/* Nanoseconds per barrier over n_groups (<= 256) co-resident workgroups that meet
+ * through device-scope loads and stores.  pattern 0: packed flags, all polled by
+ * everybody; 1: one flag per 128-byte line; 2: a tree in which every word has one
  * writer and one reader. */
 int crl_probe_barrier(int pattern, int n_groups, int rounds, double* ns_per_barrier);
 

@@ -135,8 +135,7 @@ def test_fused_fast_loop_matches_oracle(gpu, oracle, variant, N, W, H, T, steps,
         eng.run_fused(steps - steps // 2)
         q, st = eng.q_get(0, N), eng.get_state()
         hbm, lds = eng.fused_split()
-    if "hbm+lds" in info["name"] or True:
-        assert hbm + lds == N
+    assert hbm + lds == N
     Q = np.zeros((N, S, 4), np.float32)
     ost = oracle.new_state(cfg, start)
     oracle.run(cfg, cls, None, start, Q, ost, t_odd, steps)
@@ -388,9 +387,13 @@ def test_shared_table_one_launch_kernel_shapes(gpu, oracle):
     cfg = gpu.make_config(300, 16, 16, table_mode=gpu.TABLE_SHARED, map_mode=gpu.MAP_SHARED, lr=0.01, eps0=0.3,
                           episode_len=25, seed=3, trap_reward=-0.5)
     with gpu.Engine(cfg, 0) as eng:
+        # automatic: the one-launch kernel unless the call is too short to repay its set-up
+        assert eng.fused_kernel_info(10)["name"] == "k_shared_persist<4,1>"
+        assert eng.fused_kernel_info(1)["name"] == "k_shared_act+k_reduce_owners"
+        eng.set_fused_variant(1)
         assert eng.fused_kernel_info(10)["name"] == "k_shared_act+k_reduce_owners"
         eng.set_fused_variant(2)
-        assert eng.fused_kernel_info(10)["name"] == "k_shared_persist<4,1>" and eng.fused_kernel_info(10)["grid"] == 16
+        assert eng.fused_kernel_info(1)["name"] == "k_shared_persist<4,1>" and eng.fused_kernel_info(1)["grid"] == 16
     run_both(gpu, oracle, cfg, cls, start, 90, chunks=[1, 30, 1, 1, 50, 7], variant=2)
     # 8 actions, cell rewards, per-env maps (global memory), linear epsilon, 1000 envs: last block 232 envs
     N, W, H = 1000, 24, 20
@@ -438,9 +441,11 @@ def test_shared_table_one_launch_kernel_shapes(gpu, oracle):
 
 def test_shared_table_one_launch_kernel_gives_up_cleanly(gpu):
     """Failure handling of the one-launch kernel, forced from the host: with a wait of
-    one poll the workgroups do not find their peers' flags, give up, and every one of
-    them leaves the kernel; the next synchronising call reports it, and the device is
-    fine afterwards."""
+    one poll the threads do not find their peers' data, give up, and every workgroup
+    leaves the kernel.  A second call before anybody has looked must not hide the first
+    one's report (its launch sees the give-up word and returns at once); the next
+    synchronising call reports it once, calls that work on state or table are refused
+    until they are set again, and the device is fine afterwards."""
     N, W, H = 20000, 32, 32
     cls, start = gpu.gen_maps_bernoulli(6, 1, N, W, H, 0.15)
     cfg = gpu.make_config(N, W, H, table_mode=gpu.TABLE_SHARED, map_mode=gpu.MAP_SHARED, lr=0.004, eps0=0.2, seed=21)
@@ -449,10 +454,23 @@ def test_shared_table_one_launch_kernel_gives_up_cleanly(gpu):
         eng.set_fused_variant(2)
         eng.set_persist_spin_limit(1)
         eng.run_fused(50)  # asynchronous: the launch itself succeeds
+        eng.run_fused(5)   # and so does this one, on top of what the first left
         with pytest.raises(gpu.CrlError) as err:
             eng.sync()
         assert err.value.code == -2 and "gave up" in str(err.value)
         eng.sync()  # reported once
+        for call in (lambda: eng.run_fused(3), eng.get_state, lambda: eng.q_get(0), eng.select):
+            with pytest.raises(gpu.CrlError) as err:
+                call()
+            assert err.value.code == gpu.E_STATE and "gave up earlier" in str(err.value)
+        # state and table set again: the engine works, on the default wait
+        eng.set_persist_spin_limit(1 << 20)
+        eng.reset()
+        eng.q_set(0, np.zeros((W * H, 4), np.float32))
+        eng.set_state(s=start.copy(), ep_step=np.zeros(N, np.int32), episode=np.zeros(N, np.int32))
+        eng.step_count = 0
+        eng.run_fused(50)
+        q_again = eng.q_get(0)
     with gpu.Engine(cfg, 0) as eng:  # same device, default limit: all is well
         eng.set_maps(cls, start)
         eng.set_fused_variant(2)
@@ -460,8 +478,10 @@ def test_shared_table_one_launch_kernel_gives_up_cleanly(gpu):
         q_one = eng.q_get(0)
     with gpu.Engine(cfg, 0) as eng:
         eng.set_maps(cls, start)
+        eng.set_fused_variant(1)
         eng.run_fused(50)
         assert np.array_equal(eng.q_get(0), q_one) and np.isfinite(q_one).all()
+    assert np.array_equal(q_again, q_one)
 
 
 def test_shared_table_all_envs_on_one_cell(gpu, oracle):
