@@ -39,7 +39,7 @@ WORKLOADS = {
     # bytes: algorithmic bytes per env-step = 22 B of state/outputs + (4A+4) B of table
     # traffic (one new row, one write) + S/(8T) B of map per episode (+4 B/cell reward)
     # launch_steps: env-steps every env takes in one pass (the configuration's own length)
-    "c2": dict(n=4096, launch_steps=10000, bytes=42.5,
+    "c2": dict(n=4096, launch_steps=10000, bytes=42.5, traffic=8.2,
                name="c2: 4096 envs 32x32, per-env tables 1024x4, eps 0.1, T=256, 10000 steps"),
     "c3": dict(n=65536, launch_steps=1000, bytes=24.0,
                name="c3: 65536 envs, shared 64x64 map, one shared table 4096x4, ordered reduction, "
@@ -49,11 +49,12 @@ WORKLOADS = {
     "c3f": dict(n=65536, launch_steps=1000, bytes=24.0,
                 name="c3 with lr 0.0005 (finite table): 65536 envs, shared 64x64 map, one shared "
                      "table 4096x4, ordered reduction, 1000 steps"),
-    # traffic: HBM bytes per env-step from rocprofv3 FETCH_SIZE x2.000 + WRITE_SIZE x1.000
-    # (profiles/k_fused_tickets_c4.md), valid for the default launch only
-    "c4": dict(n=1 << 20, launch_steps=1000, bytes=42.25, traffic=29.8,
+    # traffic: bytes per env-step past the L2, from rocprofv3 FETCH_SIZE x2.000 + WRITE_SIZE x1.000
+    # in separate --pmc runs of the same launches (profiles/*.md), valid for the
+    # workload's own launch length only (traffic_short: c4 at 20 steps per launch)
+    "c4": dict(n=1 << 20, launch_steps=1000, bytes=42.25, traffic=29.8, traffic_short={20: 58.1},
                name="c4: 1048576 envs 16x16, per-env tables 256x4 (4 GB), traps, eps 0.1, T=128, 1000 steps"),
-    "c5": dict(n=8192, launch_steps=1024, bytes=70.0, traffic=None,
+    "c5": dict(n=8192, launch_steps=1024, bytes=70.0, traffic=87.1,
                name="c5: 8192 envs 256x256, 8 actions, per-env tables 65536x8 (16 GB), cell rewards, "
                     "eps 1.0->0.05 over 100 episodes, T=1024, 1024 steps"),
 }
@@ -224,7 +225,7 @@ def time_cpu(orc, key, n_sample, steps, threads):
         t0 = time.perf_counter()
         orc.run(cfg, cls, cr, start, Q, st, 0, steps)
         dt = time.perf_counter() - t0
-        return n_sample * steps / dt, 1, dt
+        return n_sample * steps / dt, 1, dt, (Q, st)
     Q = np.zeros((n_sample, S, A), np.float32)
     Q.fill(0.0)  # pages touched before the clock starts
     p = Oracle._p
@@ -243,11 +244,45 @@ def time_cpu(orc, key, n_sample, steps, threads):
     for t in ths:
         t.join()
     dt = time.perf_counter() - t0
-    return n_sample * steps / dt, threads, dt
+    return n_sample * steps / dt, threads, dt, (Q, st)
+
+
+def parity_check(key, n, steps, want):
+    """One launch of `steps` env-steps for the first `n` envs of the workload from its
+    initial state, on a fresh engine, against what the CPU port computed from the same
+    seeds: every state array and every table (fetched in chunks), bit for bit."""
+    Q, ost = want
+    cfg, cls, start, cr = build_workload(key, n)
+    n_tables = Q.shape[0]
+    bad = {}
+    with pycrl.Engine(cfg, 0) as eng:
+        eng.set_maps(cls, start, cr)
+        del cls, cr
+        name = eng.fused_kernel_info(steps)["name"]
+        eng.run_fused(steps)
+        st = eng.get_state()
+        for k in ("s", "ep_step", "episode", "reward", "done", "action"):
+            d = int(np.count_nonzero(st[k] != ost[k]))
+            if d:
+                bad[k] = d
+        chunk = max(1, min(n_tables, (256 << 20) // (Q[0].size * 4)))
+        bad_tables = 0
+        for lo in range(0, n_tables, chunk):
+            c = min(chunk, n_tables - lo)
+            q = eng.q_get(lo, c).reshape((c,) + Q.shape[1:])
+            bad_tables += int(c - np.count_nonzero(np.equal(q, Q[lo:lo + c]).all(axis=(1, 2)) |
+                                                   ((np.isnan(q) == np.isnan(Q[lo:lo + c])).all(axis=(1, 2)) &
+                                                    np.equal(np.nan_to_num(q), np.nan_to_num(Q[lo:lo + c])).all(axis=(1, 2)))))
+        if bad_tables:
+            bad["tables"] = bad_tables
+    return {"parity_checked": not bad, "envs": n, "env_steps_each": steps, "tables": n_tables, "kernel": name,
+            "compared": "s, ep_step, episode, reward, done, action of every env and every table entry, "
+                        "against the CPU port from the same seeds", "mismatches": bad}
 
 
 def cpu_baseline(key, full_n):
-    """Single-thread and all-threads figures of the CPU port on this host."""
+    """Single-thread and all-threads figures of the CPU port on this host, and the parity of
+    one GPU launch with what the port computed."""
     orc, flags = _native_oracle()
     nproc = os.cpu_count() or 1
     try:
@@ -260,7 +295,7 @@ def cpu_baseline(key, full_n):
     threads = max(1, min(usable, share) if share > 0 else usable)
     steps = {"c2": 10000, "c3": 1000, "c3f": 1000, "c4": 1000, "c5": 1024}[key]
     n1 = {"c2": 256, "c3": full_n, "c3f": full_n, "c4": 65536, "c5": 128}[key]
-    v1, _, dt1 = time_cpu(orc, key, min(n1, full_n), steps, 1)
+    v1, _, dt1, res1 = time_cpu(orc, key, min(n1, full_n), steps, 1)
     out = {"unit": "env-steps/s", "kind": "port", "nproc": nproc, "cpu_model": _cpu_model(),
            "compiler_flags": "gcc " + flags,
            "single_thread": {"value": v1, "cores": 1,
@@ -268,14 +303,25 @@ def cpu_baseline(key, full_n):
     if WORKLOADS[key]["name"].startswith("c3"):
         out.update(value=v1, cores=1, sample=out["single_thread"]["sample"] +
                    " (one shared table: the port's ordered reduction is serial)")
+        out["parity"] = parity_check(key, min(n1, full_n), steps, res1)
         return out
+    del res1
     # all threads: the full configuration when that is about 10 s of wall time, else a share of it
     n_all = int(min(full_n, max(threads * 64, v1 * threads * 10.0 / steps)))
-    va, cores, dta = time_cpu(orc, key, n_all, steps, threads)
+    va, cores, dta, res = time_cpu(orc, key, n_all, steps, threads)
     out.update(value=va, cores=cores,
                sample="%d of %d envs x %d steps of the same workload, %.1f s wall on %d threads"
                       % (n_all, full_n, steps, dta, cores))
+    out["parity"] = parity_check(key, n_all, steps, res)
     return out
+
+
+def measured_traffic(key, launch_steps=None):
+    """bytes per env-step past the L2 from the rocprofv3 runs under profiles/, or None"""
+    wl = WORKLOADS[key]
+    if launch_steps and launch_steps != wl["launch_steps"]:
+        return wl.get("traffic_short", {}).get(launch_steps)
+    return wl.get("traffic")
 
 
 def side_figure(key, reps, warm, launch_steps=None):
@@ -283,7 +329,12 @@ def side_figure(key, reps, warm, launch_steps=None):
     name = WORKLOADS[key]["name"]
     if launch_steps:
         name = name.rsplit(",", 1)[0] + ", %d steps per launch" % launch_steps
+    traffic = measured_traffic(key, launch_steps)
+    med_s = statistics.median(r["rep_ms"]) * 1e-3
     return {"workload": name, "value": r["steps_per_s"], "unit": "env-steps/s",
+            "value_at_median_launch": r["n"] * r["launch_steps"] / med_s,
+            "traffic_bytes_per_env_step": traffic,
+            "hbm_measured_frac": None if traffic is None else traffic * r["n"] * r["launch_steps"] / med_s / 1e9 / HBM_PEAK_GBS,
             "n_envs": r["n"], "steps_per_launch": r["launch_steps"], "launches_timed": reps,
             "us_per_env_step_round": r["device_ms"] * 1e3 / (reps * r["launch_steps"]),
             "median_launch_ms": statistics.median(r["rep_ms"]), "kernel": r["info"]["name"],
@@ -311,6 +362,8 @@ def main():
                     help="shared table, one-launch kernel: one more launch with its phase clocks armed")
     ap.add_argument("--no-cpu", action="store_true", help="skip the cpu_baseline leg")
     ap.add_argument("--no-also", action="store_true", help="skip the side measurements of the other configs")
+    ap.add_argument("--also-only", default=None, metavar="KEYS",
+                    help="comma-separated side measurements to take instead of all (c3,c3f,c2,c5)")
     args = ap.parse_args()
     if args.gpus != 1:
         raise SystemExit("bench.py: this build runs on ONE GPU (envs shard trivially, but no second "
@@ -363,26 +416,45 @@ def main():
                    "lds_bytes": g["info"]["lds_bytes"],
                    "envs_stepped_from_hbm_tables": g["split"][0], "envs_stepped_from_lds_tables": g["split"][1]},
         "roofline": {"bound": "hbm", "achieved": achieved, "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                     "frac": achieved / HBM_PEAK_GBS, "traffic": None,
+                     "frac": achieved / HBM_PEAK_GBS, "traffic": None, "hbm_measured_frac": None,
                      "algorithmic_bytes_per_env_step": wl["bytes"],
                      "algorithmic_bytes_per_launch": bytes_per_launch,
                      "kernel_ms_per_launch": avg_launch_ms},
     }
     if g["phases"]:
         out["config"]["us_per_step_by_phase"] = g["phases"]
-    if wl.get("traffic") and default_shape:
+    traffic = measured_traffic(key, args.launch_steps)
+    if traffic and not args.envs and not args.resident and not args.variant:
         # bytes past the L2 per launch, measured in separate rocprofv3 --pmc runs of this
-        # same command (profiles/), not in this run
-        out["roofline"]["traffic"] = wl["traffic"] * per_launch_units
+        # same command (profiles/), not in this run; hbm_measured_frac = that traffic over
+        # this run's launch time, as a share of the 8 TB/s peak (frac is the algorithmic-byte figure)
+        out["roofline"]["traffic"] = traffic * per_launch_units
+        out["roofline"]["hbm_measured_frac"] = traffic * per_launch_units / (avg_launch_ms * 1e-3) / 1e9 / HBM_PEAK_GBS
 
     if not args.no_cpu:
         out["cpu_baseline"] = cpu_baseline(key, g["n"])
+        out["parity_checked"] = out["cpu_baseline"]["parity"]["parity_checked"]
     if not args.no_also and not args.envs:
         also = {}
-        for k2, reps, warm in (("c3", 3, 1), ("c3f", 3, 1), ("c2", 5, 1), ("c5", 5, 1)):
-            if k2 != key:
+        only = args.also_only.split(",") if args.also_only else None
+        for k2, reps, warm in (("c3", 7, 2), ("c3f", 7, 2), ("c2", 5, 1), ("c5", 5, 1)):
+            if k2 != key and (only is None or k2 in only):
                 also[k2] = side_figure(k2, reps, warm)
-        if key == "c4" and default_shape:
+        # the target the benchmark contract names: 1e10 env-steps/s on the shared-table
+        # configuration (1-based config 3); the 0-based reading is this run's headline c4
+        c3 = also.get("c3") or (dict(value=out["value"], value_at_median_launch=out["config"]["value_at_median_launch"])
+                                if key == "c3" else None)
+        if c3:
+            ns = {"config": "c3: 65536 envs, one shared 64x64x4 table, ordered reduction, as specified",
+                  "target": 1e10, "unit": "env-steps/s", "value": c3["value_at_median_launch"],
+                  "met": c3["value_at_median_launch"] >= 1e10,
+                  "hbm_target_frac": 0.6, "hbm_measured_frac_c4": out["roofline"]["hbm_measured_frac"] if key == "c4" else None}
+            if not args.no_cpu and key != "c3":
+                orc, _ = _native_oracle()
+                _, _, dt, res = time_cpu(orc, "c3", WORKLOADS["c3"]["n"], 200, 1)
+                ns["parity"] = parity_check("c3", WORKLOADS["c3"]["n"], 200, res)
+            out["north_star"] = ns
+        if key == "c4" and default_shape and only is None:
             # what a caller that asks for a few steps at a time gets: another launch plan
             # (every env in flight, class maps staged, tables never in LDS)
             also["c4_20_steps_per_launch"] = side_figure("c4", 20, 5, 20)

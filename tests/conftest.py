@@ -205,6 +205,47 @@ def oracle_run_slice(orc, cfg, lo, hi, cls, start, t0, n_steps, cr=None):
     return Q, st
 
 
+def host_threads():
+    """Threads a test may use: the job's share of the host's cores."""
+    try:
+        usable = len(os.sched_getaffinity(0))
+    except AttributeError:
+        usable = os.cpu_count() or 1
+    share = int(os.environ.get("OMP_NUM_THREADS", "0") or 0)
+    return max(1, min(usable, share) if share > 0 else usable)
+
+
+def oracle_run_threads(orc, cfg, cls, start, t0, n_steps, cr=None, threads=None):
+    """Oracle results for ALL envs of a per-env-table batch, the envs spread over host
+    threads (they are independent, and the draws are keyed by the env index).
+    Returns (Q[N, S, A], state dict)."""
+    import threading
+    n = cfg.n_envs
+    S, A = cfg.width * cfg.height, cfg.n_actions
+    Q = np.zeros((n, S, A), np.float32)
+    st = orc.new_state(cfg, start)
+    cls = np.ascontiguousarray(cls, np.uint8)
+    start = np.ascontiguousarray(start, np.int32)
+    cr = None if cr is None else np.ascontiguousarray(cr, np.float32)
+    threads = threads or host_threads()
+    bounds = [n * i // threads for i in range(threads + 1)]
+    p = Oracle._p
+    rcs = [None] * threads
+
+    def work(i):
+        rcs[i] = orc.lib.orc_run_range(C.byref(cfg), bounds[i], bounds[i + 1], p(cls), p(cr), p(start), p(Q),
+                                       p(st["s"]), p(st["ep_step"]), p(st["episode"]), p(st["reward"]),
+                                       p(st["done"]), p(st["action"]), t0, n_steps)
+
+    ths = [threading.Thread(target=work, args=(i,)) for i in range(threads)]
+    for t in ths:
+        t.start()
+    for t in ths:
+        t.join()
+    assert rcs == [0] * threads, rcs
+    return Q, st
+
+
 @pytest.fixture(scope="session")
 def oracle():
     if not os.path.exists(ORACLE_SO):

@@ -48,6 +48,31 @@ def test_bench_prints_one_json_line_with_the_contract_keys(gpu):
     assert b["single_thread"]["cores"] == 1 and b["single_thread"]["value"] > 0
     assert b["nproc"] >= b["cores"] and isinstance(b["cpu_model"], str) and b["cpu_model"]
     assert d["value"] > b["value"]
+    # one launch on a fresh engine against what the CPU leg computed from the same seeds
+    par = b["parity"]
+    assert d["parity_checked"] is True and par["parity_checked"] is True and par["mismatches"] == {}
+    assert par["envs"] >= 64 and par["env_steps_each"] == 10000 and par["tables"] == par["envs"]
+    # measured traffic (profiles/) beside the algorithmic figure
+    assert r["traffic"] == 8.2 * c["n_envs"] * 10000
+    want = r["traffic"] / (r["kernel_ms_per_launch"] * 1e-3) / 1e9 / 8000.0
+    assert abs(r["hbm_measured_frac"] - want) <= 1e-9 * want
+
+
+@pytest.mark.gpu
+def test_bench_names_the_target_config_and_checks_it(gpu):
+    """The shared-table configuration the contract's target is quoted on: reported in a
+    `north_star` block with the target, whether it is met, and its own parity check."""
+    out = subprocess.run([sys.executable, BENCH, "--workload", "c2", "--steps", "2", "--warmup", "1",
+                          "--also-only", "c3"], capture_output=True, text=True, timeout=110)
+    assert out.returncode == 0, out.stderr
+    d = json.loads([l for l in out.stdout.splitlines() if l.strip()][-1])
+    ns = d["north_star"]
+    assert ns["target"] == 1e10 and ns["unit"] == "env-steps/s" and ns["config"].startswith("c3")
+    assert ns["met"] == (ns["value"] >= 1e10) and ns["value"] > 1e9
+    assert ns["parity"]["parity_checked"] is True and ns["parity"]["envs"] == 65536
+    c3 = d["also"]["c3"]
+    assert c3["launches_timed"] >= 5 and c3["kernel"].startswith("k_shared")
+    assert abs(ns["value"] - c3["value_at_median_launch"]) <= 1e-9 * ns["value"]
 
 
 @pytest.mark.gpu
