@@ -75,6 +75,12 @@ Array load(const std::string& path) {
   } else {
     throw std::runtime_error(path + ": unsupported .npy version");
   }
+  // the header's length is checked against the file before it is allocated
+  const std::streamoff h_at = f.tellg();
+  f.seekg(0, std::ios::end);
+  const std::streamoff h_left = f.tellg() - h_at;
+  f.seekg(h_at);
+  if (!f || h_left < 0 || hlen > (size_t)h_left) throw std::runtime_error(path + ": truncated header");
   std::string h(hlen, '\0');
   f.read(&h[0], (std::streamsize)hlen);
   if (!f) throw std::runtime_error(path + ": truncated header");
@@ -106,11 +112,10 @@ Array load(const std::string& path) {
   const size_t elem = a.is_double ? sizeof(double) : sizeof(float);
   const size_t max_elems = left > 0 ? (size_t)left / elem : 0;
   size_t n = 1;
+  for (int64_t dim : a.shape)
+    if (dim == 0) n = 0;  // an empty array, whatever the other dimensions say
   for (int64_t dim : a.shape) {
-    if (dim == 0) {
-      n = 0;
-      break;
-    }
+    if (n == 0) break;
     if (n > max_elems / (size_t)dim) throw std::runtime_error(path + ": truncated data");
     n *= (size_t)dim;
   }

@@ -11,7 +11,8 @@ import pytest
 ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
 PKG = os.path.join(ROOT, "cudarl-arena_amd")
 ORACLE_DIR = os.path.join(ROOT, "oracle")
-ORACLE_SO = os.path.join(ORACLE_DIR, "libcrl_oracle.so")
+# (CRL_ORACLE_SO: another build of the same source, e.g. the sanitized one of `make -C oracle asan`)
+ORACLE_SO = os.environ.get("CRL_ORACLE_SO") or os.path.join(ORACLE_DIR, "libcrl_oracle.so")
 
 
 def pytest_configure(config):
