@@ -125,6 +125,7 @@ struct crl_engine {
   long resident_envs = 0;  // 0 = automatic
   int fused_variant = 0;   // 0 = automatic, 1 = plain, 2 = hybrid (when it fits)
   DevBuf<unsigned> ticket;
+  DevBuf<unsigned> split;  // the engine's own copy of the last launch's ticket counters (crl_get_fused_split)
   bool hybrid_opt_in = false;
   // the scratch the call in progress works with: the engine's own allocations
   // (crl_run_fused, crl_update, crl_td_update) or the device's static array
@@ -132,6 +133,7 @@ struct crl_engine {
   bool no_alloc = false;
   unsigned char* static_scratch = nullptr;
   unsigned* tk = nullptr;  // ticket counters {next ticket, envs on HBM tables, envs on LDS tables}
+  bool split_valid = false;  // the last fused launch drew tickets
   unsigned long long* ho = nullptr;  // hand-off cells of the ordered reduction
   // one-launch shared-table kernel: what its workgroups exchange (tagged table, row
   // maxima, marks, raw samples, hand-off cells), the engine's own give-up word
@@ -182,10 +184,6 @@ struct crl_engine {
   DevBuf<int32_t> a_sup;
   uint64_t sup_t0 = 0;
   int sup_n = 0;
-  // host mirrors for crl_set_cell
-  std::vector<uint8_t> h_class;
-  std::vector<float> h_cell_reward;
-  uint32_t stage_word = 0;  // source of crl_set_cell's asynchronous one-word copy
 
   crl::Rules rules() const {
     crl::Rules R{};
@@ -733,7 +731,7 @@ int run_persist(crl_engine* e, int n_steps, bool* launched) {
     const int n = std::min(n_steps - done, crl::kPersistMaxSteps);
     const size_t w32 = p.words * 2;
     hipLaunchKernelGGL(crl::k_fill_u32, dim3((unsigned)((w32 + 255) / 256)), dim3(256), 0, e->stream,
-                       reinterpret_cast<unsigned*>(buf), 0u, (int)w32);
+                       reinterpret_cast<unsigned*>(buf), 0u, w32);
     const uint64_t t0 = e->t + (uint64_t)done;
     const int row0 = (int)std::min<long long>((long long)e->trace_cursor + done, e->trace_cap);
     hipError_t h;
@@ -838,17 +836,24 @@ int build_moves(crl_engine* e, int first, int count) {
   return CRL_OK;
 }
 
-int upload_maps(crl_engine* e) {
-  std::vector<uint32_t> packed((size_t)e->n_maps * e->map_words, 0u);
-  for (int m = 0; m < e->n_maps; ++m)
-    crl::pack_classes(e->h_class.data() + (size_t)m * e->S, e->S,
-                      packed.data() + (size_t)m * e->map_words);
-  HIP_TRY(hipMemcpyAsync(e->map.p, packed.data(), packed.size() * sizeof(uint32_t),
-                         hipMemcpyHostToDevice, e->stream));
+// Packs the caller's class maps 2 bits to a cell and uploads them a slice of maps at a
+// time (the engine keeps no host copy of maps or cell rewards: for 8192 maps of 256x256
+// cells those would be 0.5 GB and 2 GB for the life of the engine).
+int upload_maps(crl_engine* e, const uint8_t* cell_class, const float* cell_reward) {
+  const size_t slice_maps = std::max<size_t>(1, ((size_t)16 << 20) / ((size_t)e->map_words * 4));
+  std::vector<uint32_t> packed(std::min<size_t>(slice_maps, (size_t)e->n_maps) * e->map_words);
+  for (size_t m0 = 0; m0 < (size_t)e->n_maps; m0 += slice_maps) {
+    const size_t count = std::min(slice_maps, (size_t)e->n_maps - m0);
+    std::fill(packed.begin(), packed.end(), 0u);
+    for (size_t m = 0; m < count; ++m)
+      crl::pack_classes(cell_class + (m0 + m) * e->S, e->S, packed.data() + m * e->map_words);
+    HIP_TRY(hipMemcpyAsync(e->map.p + m0 * e->map_words, packed.data(), count * e->map_words * sizeof(uint32_t),
+                           hipMemcpyHostToDevice, e->stream));
+    HIP_TRY(hipStreamSynchronize(e->stream));  // the slice buffer is filled again next round
+  }
   if (e->cfg.reward_flags & CRL_REWARD_CELLS)
-    HIP_TRY(hipMemcpyAsync(e->cell_reward.p, e->h_cell_reward.data(),
-                           e->h_cell_reward.size() * sizeof(float), hipMemcpyHostToDevice,
-                           e->stream));
+    HIP_TRY(hipMemcpyAsync(e->cell_reward.p, cell_reward, (size_t)e->n_maps * e->S * sizeof(float),
+                           hipMemcpyHostToDevice, e->stream));
   const int rc = build_moves(e, 0, e->n_maps);
   if (rc) return rc;
   HIP_TRY(hipStreamSynchronize(e->stream));
@@ -901,6 +906,7 @@ int create_engine(const crl_config* cfg, int device, crl_engine** out) {
   acc(e->tr_s2.alloc(N));
   acc(e->tr_r.alloc(N));
   acc(e->tr_done.alloc(N));
+  if (cfg->table_mode == CRL_TABLE_PER_ENV) acc(e->split.alloc(3));
   if (cfg->table_mode == CRL_TABLE_SHARED) {
     acc(e->key.alloc(N));
     acc(e->delta.alloc(N));
@@ -916,12 +922,6 @@ int create_engine(const crl_config* cfg, int device, crl_engine** out) {
   if (a != hipSuccess) {
     const int code = a == hipErrorOutOfMemory ? CRL_E_ALLOC : CRL_E_DEVICE;
     return fail(code, "device allocation failed: %s", hipGetErrorString(a));
-  }
-  try {
-    e->h_class.assign((size_t)e->n_maps * e->S, (uint8_t)CRL_CELL_FREE);
-    if (cells) e->h_cell_reward.assign((size_t)e->n_maps * e->S, cfg->step_reward);
-  } catch (const std::bad_alloc&) {
-    return fail(CRL_E_ALLOC, "host allocation failed");
   }
   auto bail = [&](hipError_t x, const char* what) {
     return fail(CRL_E_DEVICE, "%s: %s", what, hipGetErrorString(x));
@@ -947,10 +947,14 @@ int create_engine(const crl_config* cfg, int device, crl_engine** out) {
   if ((h = hipMemcpyAsync(e->eps_tab.p, eps.data(), eps.size() * sizeof(float), hipMemcpyHostToDevice,
                           e->stream)) != hipSuccess)
     return bail(h, "upload eps table");
-  if (cells &&
-      (h = hipMemcpyAsync(e->cell_reward.p, e->h_cell_reward.data(), e->h_cell_reward.size() * 4,
-                          hipMemcpyHostToDevice, e->stream)) != hipSuccess)
-    return bail(h, "upload cell rewards");
+  if (cells) {  // until crl_set_maps: every cell pays the step reward
+    uint32_t bits;
+    std::memcpy(&bits, &cfg->step_reward, 4);
+    const size_t n = e->cell_reward.n;
+    hipLaunchKernelGGL(crl::k_fill_u32, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, e->stream,
+                       reinterpret_cast<unsigned*>(e->cell_reward.p), bits, n);
+    if ((h = hipGetLastError()) != hipSuccess) return bail(h, "fill cell rewards");
+  }
   if ((h = hipStreamSynchronize(e->stream)) != hipSuccess) return bail(h, "sync");
   // set-up that crl_run_fused_noalloc must not have left to do: this device's copy
   // of the scratch array, and the kernels that may use the whole LDS
@@ -991,9 +995,7 @@ int set_maps(crl_engine* e, const uint8_t* cell_class, const int32_t* start,
     for (int i = 0; i < e->N; ++i)
       if (start[i] < 0 || (size_t)start[i] >= e->S)
         return fail(CRL_E_RANGE, "start[%d] = %d outside [0,%zu)", i, start[i], e->S);
-  std::memcpy(e->h_class.data(), cell_class, total);
-  if (cells) std::memcpy(e->h_cell_reward.data(), cell_reward, total * sizeof(float));
-  rc = upload_maps(e);
+  rc = upload_maps(e, cell_class, cell_reward);
   if (rc) return rc;
   if (start) {
     HIP_TRY(hipMemcpyAsync(e->start.p, start, (size_t)e->N * 4, hipMemcpyHostToDevice, e->stream));
@@ -1010,21 +1012,19 @@ int set_cell(crl_engine* e, int32_t map_index, int32_t cell, int32_t cell_class,
   if (cell < 0 || (size_t)cell >= e->S) return fail(CRL_E_RANGE, "cell %d outside [0,%zu)", cell, e->S);
   if (cell_class < CRL_CELL_FREE || cell_class > CRL_CELL_WALL) return fail(CRL_E_ARG, "%d is not a cell class", cell_class);
   const size_t at = (size_t)map_index * e->S + cell;
-  e->h_class[at] = (uint8_t)cell_class;
+  // the word of 16 cells that holds this one: fetched, changed, put back
   const size_t word = (size_t)map_index * e->map_words + (cell >> 4);
-  uint32_t& packed = e->stage_word;  // outlives this call: the copy below is asynchronous
-  packed = 0;
-  const size_t first = (size_t)map_index * e->S + ((size_t)(cell >> 4) << 4);
-  for (size_t j = 0; j < 16 && ((size_t)(cell >> 4) << 4) + j < e->S; ++j)
-    packed |= (uint32_t)(e->h_class[first + j] & 3u) << (2 * j);
+  uint32_t packed = 0;
+  HIP_TRY(hipMemcpyAsync(&packed, e->map.p + word, 4, hipMemcpyDeviceToHost, e->stream));
+  HIP_TRY(hipStreamSynchronize(e->stream));
+  const int shift = 2 * (cell & 15);
+  packed = (packed & ~(3u << shift)) | ((uint32_t)cell_class << shift);
   HIP_TRY(hipMemcpyAsync(e->map.p + word, &packed, 4, hipMemcpyHostToDevice, e->stream));
   rc = build_moves(e, map_index, 1);  // the neighbours' codes name this cell
   if (rc) return rc;
-  if (e->cfg.reward_flags & CRL_REWARD_CELLS) {
-    e->h_cell_reward[at] = cell_reward;
-    HIP_TRY(hipMemcpyAsync(e->cell_reward.p + at, &e->h_cell_reward[at], 4, hipMemcpyHostToDevice, e->stream));
-  }
-  HIP_TRY(hipStreamSynchronize(e->stream));
+  if (e->cfg.reward_flags & CRL_REWARD_CELLS)
+    HIP_TRY(hipMemcpyAsync(e->cell_reward.p + at, &cell_reward, 4, hipMemcpyHostToDevice, e->stream));
+  HIP_TRY(hipStreamSynchronize(e->stream));  // `packed` and `cell_reward` are this call's
   return CRL_OK;
 }
 
@@ -1088,6 +1088,12 @@ int run_fused(crl_engine* e, int32_t n_steps, bool no_alloc) {
     else
       launch_fused_a<8>(e, p, e->t, n_steps);
     HIP_TRY(hipGetLastError());
+    if (p.tickets) {
+      // the counters may sit in the scratch all engines of this GPU share: kept here
+      hipLaunchKernelGGL(crl::k_copy3_u32, dim3(1), dim3(64), 0, e->stream, e->tk, e->split.p);
+      HIP_TRY(hipGetLastError());
+    }
+    e->split_valid = p.tickets;
     if (e->trace_n > 0) {
       const long long c = (long long)e->trace_cursor + n_steps;
       e->trace_cursor = c > e->trace_cap ? e->trace_cap : (int)c;
@@ -1160,8 +1166,8 @@ int crl_get_fused_split(crl_engine* e, uint32_t* hbm_envs, uint32_t* lds_envs) {
   int rc = check_usable(e);
   if (rc) return rc;
   unsigned v[3] = {0, 0, 0};
-  if (e->tk) {
-    HIP_TRY(hipMemcpyAsync(v, e->tk, sizeof v, hipMemcpyDeviceToHost, e->stream));
+  if (e->split_valid) {
+    HIP_TRY(hipMemcpyAsync(v, e->split.p, sizeof v, hipMemcpyDeviceToHost, e->stream));
     HIP_TRY(hipStreamSynchronize(e->stream));
   }
   if (hbm_envs) *hbm_envs = v[1];

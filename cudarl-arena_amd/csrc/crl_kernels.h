@@ -1012,9 +1012,13 @@ __global__ __launch_bounds__(256) void k_build_moves(const uint32_t* __restrict_
   moves[(size_t)m * mv_words + w] = out;
 }
 
-__global__ void k_fill_u32(unsigned* p, const unsigned v, const int n) {
-  const int i = blockIdx.x * blockDim.x + threadIdx.x;
+__global__ void k_fill_u32(unsigned* p, const unsigned v, const size_t n) {
+  const size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
   if (i < n) p[i] = v;
+}
+// (a launch instead of a device-to-device copy: a caller may record the call)
+__global__ void k_copy3_u32(const unsigned* __restrict__ src, unsigned* __restrict__ dst) {
+  if (threadIdx.x < 3) dst[threadIdx.x] = src[threadIdx.x];
 }
 
 // plain copy of n16 16-byte words: the known-size launch that calibrates the
