@@ -216,15 +216,25 @@ __device__ __forceinline__ bool reduce_block(ReduceLds& L, const ReduceGeom G, c
   const bool over = L.over != 0;
 
   if (DEV) {
+    // (256 owners x 4 pieces = four pieces to a thread, all asked for before the first is used)
     const ulonglong2* stage2 = reinterpret_cast<const ulonglong2*>(stage);
-    for (int i = tid; i < n_own * (kHandoffRecs / 2); i += kBlockSamples) {
-      ulonglong2 v = stage2[i];
-      if ((i & 3) == 0) {
-        const int c = L.handed[i >> 2];
-        v.x |= (unsigned long long)(uint32_t)(c > kSlotCap ? kSlotOverflow : c) << kRecCountShift;
-      }
-      st_dev128(*window, window_offset + (uint32_t)(((size_t)block * n_own * kHandoffRecs + (size_t)i * 2) * 8),
-                make_uint4((uint32_t)v.x, (uint32_t)(v.x >> 32), (uint32_t)v.y, (uint32_t)(v.y >> 32)));
+    const int pieces = n_own * (kHandoffRecs / 2);
+    constexpr int kPer = (256 * (kHandoffRecs / 2)) / kBlockSamples;
+    ulonglong2 v[kPer];
+    int c[kPer];
+#pragma unroll
+    for (int j = 0; j < kPer; ++j) {
+      const int i = tid + j * kBlockSamples;
+      v[j] = i < pieces ? stage2[i] : make_ulonglong2(0ull, 0ull);
+      c[j] = (i < pieces && (i & 3) == 0) ? L.handed[i >> 2] : 0;
+    }
+#pragma unroll
+    for (int j = 0; j < kPer; ++j) {
+      const int i = tid + j * kBlockSamples;
+      v[j].x |= (unsigned long long)(uint32_t)(c[j] > kSlotCap ? kSlotOverflow : c[j]) << kRecCountShift;
+      if (i < pieces)
+        st_dev128(*window, window_offset + (uint32_t)(((size_t)block * n_own * kHandoffRecs + (size_t)i * 2) * 8),
+                  make_uint4((uint32_t)v[j].x, (uint32_t)(v[j].x >> 32), (uint32_t)v[j].y, (uint32_t)(v[j].y >> 32)));
     }
   } else {
     if (leader && slot < kSlotCap) {
