@@ -277,7 +277,7 @@ struct FusedPlan {
   bool hybrid;     // ... whose last wave per workgroup steps envs whose tables it holds in LDS
   bool fast;       // the folded loop for the common configuration
   bool moves;      // ... whose table waves read pre-built move codes from LDS
-  bool fixed;      // every pair of tickets has its own wave: dealt by position, no counter
+  bool fixed;      // tickets dealt by position, round after round: no counter
   bool pair;       // per-env kernel: two lanes per env
   int pair_envs;   // ticket kernel: envs per thin table wave (32, 16, 8), 0: 64-env waves
   bool rich;       // ticket kernel: the folded loop's variant with per-cell rewards / per-episode epsilon
@@ -419,7 +419,11 @@ FusedPlan plan_fused(const crl_engine* e, int n_steps) {
         units = (e->N + p.pair_envs - 1) / p.pair_envs;
         p.grid = (int)std::min<long>(std::max<long>(1, resident / p.pair_envs), units);
       }
-      p.fixed = (long)p.grid * waves * (p.pair ? 1 : 2) >= units && n_steps < kHybridMinSteps;  // a wave for every pair of tickets
+      // Tickets dealt by position instead of drawn from a counter: the workers of this plan
+      // all take the same time, and 16,384 draws from one counter take 0.38 ms however short
+      // the launch (1M envs: the whole of a 4-step launch, half of a 20-step one).
+      p.fixed = n_steps < kHybridMinSteps;
+      (void)units;
       p.lds = waves * (p.moves ? mv_lds : map_lds);
     }
   }

@@ -594,17 +594,19 @@ __global__ __launch_bounds__(LDSW ? 320 : 256) void k_fused_tickets(const Rules 
   const unsigned take = thin ? 1u : 2u;
   const size_t table = P.S * A;  // floats per table
 
-  // With a wave for every pair of tickets (fixed_tickets: a short launch with all
+  // fixed_tickets: the tickets are dealt by position, wave after wave, round after round
+  // (workers that all take the same time need no counter).  With a wave for every pair of tickets (a short launch with all
   // envs in flight) the tickets are dealt by position: tens of thousands of
   // atomic draws from one counter would take longer than the few steps.
   if (fixed_tickets && blockIdx.x == 0 && threadIdx.x == 0) {
     ticket[1] = (unsigned)P.N;
     ticket[2] = 0u;
   }
-  for (bool first = true;; first = false) {
+  unsigned stepped = 0;  // envs this worker has stepped
+  for (unsigned round = 0;; ++round) {
     unsigned base = 0;
     if (fixed_tickets) {
-      base = first ? (blockIdx.x * (unsigned)n_waves + (unsigned)wave) * take : n_tickets;
+      base = ((round * gridDim.x + blockIdx.x) * (unsigned)n_waves + (unsigned)wave) * take;
     } else {
       if (lane == 0) base = atomicAdd(ticket, take);
       base = __shfl(base, 0);
@@ -614,7 +616,7 @@ __global__ __launch_bounds__(LDSW ? 320 : 256) void k_fused_tickets(const Rules 
     const int n_here = min(cap, P.N - env0);
     const int env = env0 + lane;
     const bool live = lane < n_here;
-    if (!fixed_tickets && lane == 0) atomicAdd(ticket + (lds_worker ? 2 : 1), (unsigned)n_here);  // who did how much
+    stepped += (unsigned)n_here;
 
     // this worker's maps: contiguous in HBM, transposed into [word][lane]
     __builtin_amdgcn_wave_barrier();
@@ -711,6 +713,9 @@ __global__ __launch_bounds__(LDSW ? 320 : 256) void k_fused_tickets(const Rules 
       for (int i = j0 + lane; i < total4; i += 64) stream_store4(get(i), o4 + i);
     }
   }
+  // who did how much: once per worker (a pair of atomics per ticket had every wave of a
+  // short launch queue at the counters whenever a round of tickets ended)
+  if (!fixed_tickets && lane == 0 && stepped != 0u) atomicAdd(ticket + (lds_worker ? 2 : 1), stepped);
 }
 
 // ---------------------------------------------------------------------------
