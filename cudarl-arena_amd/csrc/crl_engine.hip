@@ -507,11 +507,12 @@ crl::ReduceGeom reduce_geom(const crl_engine* e, int n) {
   G.a_shift = e->A == 8 ? 3 : 2;
   G.own_shift = ceil_log2((e->K + crl::kOwnKeys - 1) / crl::kOwnKeys);
   G.n_blocks = (n + crl::kBlockSamples - 1) / crl::kBlockSamples;
+  G.cell_shift = crl::cell_shift_for(G.own_shift);
   return G;
 }
 
 size_t handoff_records(const crl::ReduceGeom& G) {
-  return ((size_t)1 << G.own_shift) * (size_t)G.n_blocks * crl::kHandoffRecs;
+  return (((size_t)1 << G.own_shift) * (size_t)G.n_blocks) << G.cell_shift;
 }
 
 // the two-pass reduction needs the dense LDS table (K <= 16384) and a bounded hand-off buffer
@@ -673,6 +674,9 @@ PersistPlan plan_persist(const crl_engine* e, int n_steps) {
   const int n_own = 1 << p.G.own_shift;
   p.grid = std::max(n_blocks, n_own);
   if (e->K > (size_t)crl::kDenseKeys || p.grid > crl::kPersistMaxGroups || p.grid > kComputeUnits) return p;
+  // (few owners have large hand-off cells, fetched eight loads at a time; 65,536 envs on a
+  // 16x16x4 table: 14.5 us per step in one launch, 10.3 with two launches per step)
+  if (e->fused_variant == 0 && p.G.cell_shift > 4) return p;
   p.G.n_blocks = p.grid;  // workgroups without envs hand over empty cells
   const size_t map_bytes = (size_t)e->map_words * 4;
   p.lds_map = e->cfg.map_mode == CRL_MAP_SHARED && sizeof(crl::PersistLds) + map_bytes <= kLdsPerWorkgroup - kStaticLdsReserve;
@@ -683,7 +687,7 @@ PersistPlan plan_persist(const crl_engine* e, int n_steps) {
   p.at_mark = p.at_rowmax + pad(e->S);
   p.at_raw = p.at_mark + pad((size_t)n_own);
   p.at_cells = p.at_raw + pad(2 * (size_t)e->N);  // raw samples and cells: two buffers each
-  p.words = p.at_cells + 2 * (size_t)n_own * p.grid * crl::kHandoffRecs;
+  p.words = p.at_cells + 2 * (((size_t)n_own * p.grid) << p.G.cell_shift);
   if (e->no_alloc && p.words * sizeof(unsigned long long) > kScratchExchangeBytes) return p;
   p.ok = true;
   return p;

@@ -37,6 +37,8 @@
 // Every wait is bounded: a thread that polls `spin_limit` times in vain (or sees the
 // give-up word set) makes its workgroup set the give-up word and leave.
 #pragma once
+#include <type_traits>
+
 #include "crl_kernels.h"
 
 namespace crl {
@@ -156,7 +158,7 @@ __global__ __launch_bounds__(256) void k_shared_persist(const Rules R, const Ptr
   const uint32_t* gmap = P.map + ((P.map_shared || !has_env) ? 0 : (size_t)env * P.map_words);
   const float* cr = P.cell_reward ? P.cell_reward + ((P.map_shared || !has_env) ? 0 : (size_t)env * P.S) : nullptr;
   const DevWindow w_table = dev_window(B.table), w_cells = dev_window(B.cells);
-  const size_t cells_half = (size_t)n_own * G.n_blocks * kHandoffRecs;  // 64-bit words of one buffer of cells
+  const size_t cells_half = ((size_t)n_own * G.n_blocks) << G.cell_shift;  // 64-bit words of one buffer of cells
   const bool cells_flag = (R.reward_flags & 1) != 0;
   const bool base_cells = cells_flag && (R.reward_flags & 2) != 0;
 
@@ -359,66 +361,81 @@ __global__ __launch_bounds__(256) void k_shared_persist(const Rules R, const Ptr
 
     // ---- as owner of 64 keys: all blocks' cells, added in tree order --------------------
     if (is_owner) {
-      // A wave takes 64 blocks' cells: 4 KB that it reads side by side, 16 bytes = two
-      // records to a lane and load, so that a load of the wave is a handful of whole
-      // lines instead of 64 pieces of 64 different lines.  Lanes 4c .. 4c+3 of load j hold
-      // the eight records of block 64 * wave + 16 * j + c.
-      uint4 rec[4];
-      int cnt[4];
+      // A wave takes 64 blocks' cells, 16 bytes = two records to a lane and load: the
+      // lanes that share a cell (4 for cells of eight records, up to 32) read it side by
+      // side, so a load of the wave is whole cells instead of 64 pieces of 64 different
+      // ones.  GS loads at a time are asked for, checked and put into the tile: all four
+      // of cells of eight records, eight at a time of larger cells.
       {
-        const int pair = lane & 3;
-        uint32_t src[4];  // byte offsets into the cells
-        bool have[4];
+        const int pc_shift = G.cell_shift - 1;            // log2(pieces of a cell)
+        const int pair = lane & ((1 << pc_shift) - 1);    // this lane's piece of its cell
+        const int cells_per_load = 64 >> pc_shift;
+        const int n_loads = 1 << pc_shift;
+        auto fetch_cells = [&](auto group_size) {
+          constexpr int GS = decltype(group_size)::value;
+          int spins = 0;
+          bool stop = false;
+          for (int j0 = 0; j0 < n_loads && !stop; j0 += GS) {
+            uint4 rec[GS];
+            int cnt[GS];
+            uint32_t src[GS];  // byte offsets into the cells
+            bool have[GS];
 #pragma unroll
-        for (int j = 0; j < 4; ++j) {
-          const int blk = wave * 64 + j * 16 + (lane >> 2);
-          have[j] = blk < G.n_blocks;
-          src[j] = (uint32_t)(((size_t)half * cells_half + (size_t)((have[j] ? blk : 0) * n_own + wg) * kHandoffRecs + 2 * pair) * 8);
-        }
-        bool ok = false;
-        int spins = 0;
-        for (;;) {
-          poll_fence();
+            for (int j = 0; j < GS; ++j) {
+              const int blk = wave * 64 + (j0 + j) * cells_per_load + (lane >> pc_shift);
+              have[j] = blk < G.n_blocks;
+              src[j] = (uint32_t)(((size_t)half * cells_half + ((size_t)((have[j] ? blk : 0) * n_own + wg) << G.cell_shift) + 2 * pair) * 8);
+            }
+            for (;;) {
+              poll_fence();
 #pragma unroll
-          for (int j = 0; j < 4; ++j) rec[j] = ld_dev128(w_cells, src[j]);
-          ok = true;
+              for (int j = 0; j < GS; ++j) rec[j] = ld_dev128(w_cells, src[j]);
+              bool ok = true;
 #pragma unroll
-          for (int j = 0; j < 4; ++j) {
-            const uint32_t meta0 = (uint32_t)__shfl((int)rec[j].x, lane & ~3);
-            const int c = rec_count(meta0);
-            cnt[j] = c;
-            // (every record of a cell is written every step)
-            const bool mine = rec_tag(meta0) == want && rec_tag(rec[j].x) == want && rec_tag(rec[j].z) == want;
-            ok = ok && (mine || !have[j]);
-          }
-          if (__all(ok)) break;
-          if (++spins >= spin_limit || ((spins & 63) == 0 && ld_dev32(B.err) != 0u)) {
-            L.dead = 1;
-            break;
-          }
-        }
-        if (CLK) phase_[9] += (unsigned long long)spins + 1ull;
-        __syncthreads();  // (also: the tile is clear for everybody)
-        if (L.dead) {
-          gave_up = true;
-          break;
-        }
+              for (int j = 0; j < GS; ++j) {
+                const uint32_t meta0 = (uint32_t)__shfl((int)rec[j].x, lane - pair);
+                cnt[j] = rec_count(meta0);
+                // (every record of a cell is written every step)
+                const bool mine = rec_tag(meta0) == want && rec_tag(rec[j].x) == want && rec_tag(rec[j].z) == want;
+                ok = ok && (mine || !have[j]);
+              }
+              if (__all(ok)) break;
+              if (++spins >= spin_limit || ((spins & 63) == 0 && ld_dev32(B.err) != 0u)) {
+                L.dead = 1;
+                stop = true;
+                break;
+              }
+            }
+            if (j0 == 0) {
+              if (CLK) phase_[9] += (unsigned long long)spins + 1ull;
+              __syncthreads();  // the tile is clear for everybody
+              stop = stop || L.dead != 0;
+            }
+            if (stop) break;
 #pragma unroll
-        for (int j = 0; j < 4; ++j) {
-          const int blk = wave * 64 + j * 16 + (lane >> 2);
-          if (have[j]) {
-            float* row = L.tile + blk * kOwnKeys;
-            if (cnt[j] == kSlotOverflow) {
-              if (pair == 0) L.o_list[atomicAdd(&L.o_count, 1)] = (uint8_t)blk;
-            } else {
-              if (2 * pair < cnt[j]) row[rec_slot(rec[j].x)] = __uint_as_float(rec[j].y);
-              if (2 * pair + 1 < cnt[j]) row[rec_slot(rec[j].z)] = __uint_as_float(rec[j].w);
+            for (int j = 0; j < GS; ++j) {
+              const int blk = wave * 64 + (j0 + j) * cells_per_load + (lane >> pc_shift);
+              if (have[j]) {
+                float* row = L.tile + blk * kOwnKeys;
+                if (cnt[j] == kSlotOverflow) {
+                  if (pair == 0) L.o_list[atomicAdd(&L.o_count, 1)] = (uint8_t)blk;
+                } else {
+                  if (2 * pair < cnt[j]) row[rec_slot(rec[j].x)] = __uint_as_float(rec[j].y);
+                  if (2 * pair + 1 < cnt[j]) row[rec_slot(rec[j].z)] = __uint_as_float(rec[j].w);
+                }
+              }
             }
           }
-        }
+        };
+        if (n_loads == 4) fetch_cells(std::integral_constant<int, 4>{});
+        else fetch_cells(std::integral_constant<int, 8>{});
       }
       CRL_MARK(5);
       __syncthreads();
+      if (L.dead) {  // some wave gave up waiting for its cells
+        gave_up = true;
+        break;
+      }
       // blocks with more distinct keys for this owner than a cell holds: their raw
       // samples, all threads at once, then one thread per key adds its matches in order
       const int n_over = L.o_count;

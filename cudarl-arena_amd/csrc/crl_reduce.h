@@ -25,9 +25,9 @@ namespace crl {
 constexpr int kBlockSamples = 256;   // level 0
 constexpr int kGroupBlocks = 16;     // level 1
 constexpr int kOwnKeys = 64;         // keys per owner workgroup: 64 / A whole table rows
-constexpr int kSlotCap = 8;          // block sums one block can hand one owner
-constexpr int kHandoffRecs = 8;      // one 64-byte hand-off cell of 8 records
-constexpr int kSlotOverflow = 15;    // count value: read the block's raw samples instead
+constexpr int kMinCellRecs = 8;      // records of a hand-off cell: 8 ... 64, see cell_shift_for()
+constexpr int kSlotOverflow = 127;   // count value: more distinct keys than records, read the block's raw samples instead
+constexpr int kStagePieces = 1024;   // 16-byte pieces of one block's cells at most: owners x records / 2
 constexpr int kDenseKeys = 16384;    // keys the dense LDS table of pass 1 can hold
 constexpr int kTileBlocks = 256;     // blocks per LDS tile of pass 2
 constexpr uint32_t kOwnerMix = 37;   // odd: spreads cells a power of two apart over owners
@@ -35,19 +35,19 @@ constexpr uint32_t kNoLead = 0xFFFFFFFFu;
 
 // A hand-off record is 64 bits, written and read as one unit:
 //   bits  0..5   slot of the key among its owner's 64
-//   bits  6..9   record 0 of a cell only: how many records the cell holds
-//                (0: none, kSlotOverflow: more than kSlotCap distinct keys)
-//   bits 10..31  step tag (the one-launch kernel: a record is valid once its tag is
+//   bits  6..12  record 0 of a cell only: how many records the cell holds
+//                (0: none, kSlotOverflow: more distinct keys than the cell has records)
+//   bits 13..31  step tag (the one-launch kernel: a record is valid once its tag is
 //                the step's; 0 where launches separate the steps)
 //   bits 32..63  the block sum, fp32
-constexpr int kRecCountShift = 6, kRecTagShift = 10;
+constexpr int kRecCountShift = 6, kRecTagShift = 13;
 constexpr uint32_t kRecTagMask = (1u << (32 - kRecTagShift)) - 1u;
 __device__ __forceinline__ unsigned long long make_rec(uint32_t slot, uint32_t count, uint32_t tag, float v) {
   const uint32_t meta = slot | (count << kRecCountShift) | (tag << kRecTagShift);
   return (unsigned long long)meta | ((unsigned long long)__float_as_uint(v) << 32);
 }
 __device__ __forceinline__ int rec_slot(uint32_t meta) { return (int)(meta & 63u); }
-__device__ __forceinline__ int rec_count(uint32_t meta) { return (int)((meta >> kRecCountShift) & 15u); }
+__device__ __forceinline__ int rec_count(uint32_t meta) { return (int)((meta >> kRecCountShift) & 127u); }
 __device__ __forceinline__ uint32_t rec_tag(uint32_t meta) { return meta >> kRecTagShift; }
 
 struct ReduceGeom {
@@ -55,7 +55,17 @@ struct ReduceGeom {
   int a_shift;    // log2(A)
   int own_shift;  // log2(number of owners); owners = 1 << own_shift, (K >> own_shift) <= 64
   int n_blocks;   // ceil(n / 256)
+  int cell_shift; // log2(records of a hand-off cell), cell_shift_for(own_shift)
 };
+
+// Records per hand-off cell.  A block's 256 samples spread over the owners, so a cell
+// sees about 256 / owners distinct keys: eight records for 256 owners (more than eight
+// keys once in a million cells), more where fewer owners share the samples, and all 64
+// keys an owner has from 16 owners down, where a cell cannot overflow at all.  A block's
+// cells together stay within 16 KB.
+__host__ __device__ constexpr int cell_shift_for(int own_shift) {
+  return own_shift >= 8 ? 3 : own_shift >= 6 ? 4 : own_shift == 5 ? 5 : 6;
+}
 
 // key <-> (owner, slot in the owner's 64).  An owner holds whole table rows:
 // hi = cell >> own_shift, owner = (cell + 37 * hi) mod owners, slot = hi * A + action
@@ -152,8 +162,8 @@ __device__ __forceinline__ void reduce_block_init(ReduceLds& L) {
 // out as whole lines, 16 bytes to a store and lane, every record carrying `tag`:
 // scattered 8-byte stores are partial line writes, and some 350 of them per workgroup
 // took 1.6 us to be acknowledged.  `window` is a buffer window on `handoff`.
-// Returns (to every thread) whether some owner was handed more than kSlotCap
-// distinct keys: its cell then says kSlotOverflow and the owner needs the block's
+// Returns (to every thread) whether some owner was handed more distinct keys than a
+// cell has records: its cell then says kSlotOverflow and the owner needs the block's
 // raw samples.
 // DEV = true: before each reduce_block(), separated from it by a barrier (and from the
 // one before by another): every record of every cell starts as "nothing, of this step".
@@ -162,7 +172,7 @@ __device__ __forceinline__ void reduce_block_init(ReduceLds& L) {
 __device__ __forceinline__ void reduce_stage_init(unsigned long long* stage, const ReduceGeom G, const uint32_t tag) {
   const unsigned long long none = make_rec(0u, 0u, tag, 0.0f);
   ulonglong2* stage2 = reinterpret_cast<ulonglong2*>(stage);
-  for (int i = threadIdx.x; i < (kHandoffRecs / 2) << G.own_shift; i += kBlockSamples) stage2[i] = make_ulonglong2(none, none);
+  for (int i = threadIdx.x; i < 1 << (G.cell_shift - 1 + G.own_shift); i += kBlockSamples) stage2[i] = make_ulonglong2(none, none);
 }
 
 template <bool DEV>
@@ -173,6 +183,7 @@ __device__ __forceinline__ bool reduce_block(ReduceLds& L, const ReduceGeom G, c
                                              const uint32_t window_offset = 0) {
   const int tid = threadIdx.x;
   const int n_own = 1 << G.own_shift;
+  const int cap = 1 << G.cell_shift;  // records of a cell
   if (valid) atomicMin(&L.lead[key], (uint32_t)tid);
   L.delta[tid] = delta;
   __syncthreads();
@@ -208,44 +219,45 @@ __device__ __forceinline__ bool reduce_block(ReduceLds& L, const ReduceGeom G, c
     L.lead[key] = kNoLead;
     owner = owner_of(key, G);
     slot = atomicAdd(&L.handed[owner], 1);  // slot order is free: records carry the key
-    if (slot >= kSlotCap) L.over = 1;
+    if (slot >= cap) L.over = 1;
     // (record 0's count is added on the way out, when every leader has drawn its slot)
-    if (DEV && slot < kSlotCap) stage[owner * kHandoffRecs + slot] = make_rec((uint32_t)slot_of(key, G), 0u, tag, acc);
+    if (DEV && slot < cap) stage[(owner << G.cell_shift) + slot] = make_rec((uint32_t)slot_of(key, G), 0u, tag, acc);
   }
   __syncthreads();
   const bool over = L.over != 0;
 
   if (DEV) {
-    // (256 owners x 4 pieces = four pieces to a thread, all asked for before the first is used)
+    // (at most kStagePieces pieces = four to a thread, all asked for before the first is used)
     const ulonglong2* stage2 = reinterpret_cast<const ulonglong2*>(stage);
-    const int pieces = n_own * (kHandoffRecs / 2);
-    constexpr int kPer = (256 * (kHandoffRecs / 2)) / kBlockSamples;
+    const int piece_shift = G.cell_shift - 1;  // log2(pieces of a cell)
+    const int pieces = n_own << piece_shift;
+    constexpr int kPer = kStagePieces / kBlockSamples;
     ulonglong2 v[kPer];
     int c[kPer];
 #pragma unroll
     for (int j = 0; j < kPer; ++j) {
       const int i = tid + j * kBlockSamples;
       v[j] = i < pieces ? stage2[i] : make_ulonglong2(0ull, 0ull);
-      c[j] = (i < pieces && (i & 3) == 0) ? L.handed[i >> 2] : 0;
+      c[j] = (i < pieces && (i & ((1 << piece_shift) - 1)) == 0) ? L.handed[i >> piece_shift] : 0;
     }
 #pragma unroll
     for (int j = 0; j < kPer; ++j) {
       const int i = tid + j * kBlockSamples;
-      v[j].x |= (unsigned long long)(uint32_t)(c[j] > kSlotCap ? kSlotOverflow : c[j]) << kRecCountShift;
+      v[j].x |= (unsigned long long)(uint32_t)(c[j] > cap ? kSlotOverflow : c[j]) << kRecCountShift;
       if (i < pieces)
-        st_dev128(*window, window_offset + (uint32_t)(((size_t)block * n_own * kHandoffRecs + (size_t)i * 2) * 8),
+        st_dev128(*window, window_offset + (uint32_t)((((size_t)block * n_own) << (G.cell_shift + 3)) + (size_t)i * 16),
                   make_uint4((uint32_t)v[j].x, (uint32_t)(v[j].x >> 32), (uint32_t)v[j].y, (uint32_t)(v[j].y >> 32)));
     }
   } else {
-    if (leader && slot < kSlotCap) {
+    if (leader && slot < cap) {
       uint32_t count = 0;
       if (slot == 0) {
         const int c = L.handed[owner];  // final: every leader has drawn its slot
-        count = (uint32_t)(c > kSlotCap ? kSlotOverflow : c);
+        count = (uint32_t)(c > cap ? kSlotOverflow : c);
       }
-      handoff[((size_t)block * n_own + owner) * kHandoffRecs + slot] = make_rec((uint32_t)slot_of(key, G), count, tag, acc);
+      handoff[((((size_t)block * n_own) + owner) << G.cell_shift) + slot] = make_rec((uint32_t)slot_of(key, G), count, tag, acc);
     }
-    if (tid < n_own && L.handed[tid] == 0) handoff[((size_t)block * n_own + tid) * kHandoffRecs] = make_rec(0u, 0u, tag, 0.0f);
+    if (tid < n_own && L.handed[tid] == 0) handoff[(((size_t)block * n_own) + tid) << G.cell_shift] = make_rec(0u, 0u, tag, 0.0f);
   }
   return over;
 }
@@ -285,15 +297,16 @@ __global__ __launch_bounds__(256) void k_reduce_owners(const ReduceGeom G, float
 
   for (int b0 = 0; b0 < G.n_blocks; b0 += kTileBlocks) {
     const int b = b0 + tid;
-    // the whole hand-off cell in one go: no load depends on another
-    uint4 cell[kHandoffRecs / 2];
+    // the first eight records of the hand-off cell in one go: no load depends on
+    // another (a cell with more records has the rest fetched below, when it holds them)
+    uint4 cell[kMinCellRecs / 2];
+    const uint4* src = reinterpret_cast<const uint4*>(handoff + ((((size_t)b << G.own_shift) + owner) << G.cell_shift));
     if (b < G.n_blocks) {
-      const uint4* src = reinterpret_cast<const uint4*>(handoff + ((size_t)b * (1 << G.own_shift) + owner) * kHandoffRecs);
 #pragma unroll
-      for (int i = 0; i < kHandoffRecs / 2; ++i) cell[i] = src[i];
+      for (int i = 0; i < kMinCellRecs / 2; ++i) cell[i] = src[i];
     } else {
 #pragma unroll
-      for (int i = 0; i < kHandoffRecs / 2; ++i) cell[i] = make_uint4(0, 0, 0, 0);
+      for (int i = 0; i < kMinCellRecs / 2; ++i) cell[i] = make_uint4(0, 0, 0, 0);
     }
     // the tile is cleared by all threads side by side (a thread clearing its own row
     // would put all 64 lanes of a store on the same LDS banks)
@@ -305,9 +318,14 @@ __global__ __launch_bounds__(256) void k_reduce_owners(const ReduceGeom G, float
     if (c != kSlotOverflow) {
       float* row = tile + tid * kOwnKeys;
 #pragma unroll
-      for (int i = 0; i < kHandoffRecs / 2; ++i) {
+      for (int i = 0; i < kMinCellRecs / 2; ++i) {
         if (c > 2 * i) row[rec_slot(cell[i].x)] = __uint_as_float(cell[i].y);
         if (c > 2 * i + 1) row[rec_slot(cell[i].z)] = __uint_as_float(cell[i].w);
+      }
+      for (int i = kMinCellRecs / 2; 2 * i < c; ++i) {
+        const uint4 more = src[i];
+        row[rec_slot(more.x)] = __uint_as_float(more.y);
+        if (c > 2 * i + 1) row[rec_slot(more.z)] = __uint_as_float(more.w);
       }
     } else {
       // more distinct keys than slots: redo the block's part from its samples, in order

@@ -387,9 +387,8 @@ def test_shared_table_one_launch_kernel_shapes(gpu, oracle):
     cfg = gpu.make_config(300, 16, 16, table_mode=gpu.TABLE_SHARED, map_mode=gpu.MAP_SHARED, lr=0.01, eps0=0.3,
                           episode_len=25, seed=3, trap_reward=-0.5)
     with gpu.Engine(cfg, 0) as eng:
-        # automatic: the one-launch kernel unless the call is too short to repay its set-up
-        assert eng.fused_kernel_info(10)["name"] == "k_shared_persist<4,1>"
-        assert eng.fused_kernel_info(1)["name"] == "k_shared_act+k_reduce_owners"
+        # automatic: two launches per step for a table this small (16 owners)
+        assert eng.fused_kernel_info(10)["name"] == "k_shared_act+k_reduce_owners"
         eng.set_fused_variant(1)
         assert eng.fused_kernel_info(10)["name"] == "k_shared_act+k_reduce_owners"
         eng.set_fused_variant(2)
@@ -482,6 +481,46 @@ def test_shared_table_one_launch_kernel_gives_up_cleanly(gpu):
         eng.run_fused(50)
         assert np.array_equal(eng.q_get(0), q_one) and np.isfinite(q_one).all()
     assert np.array_equal(q_again, q_one)
+
+
+def test_shared_table_automatic_plan_and_cell_sizes(gpu, oracle):
+    """What crl_run_fused picks by itself, and the hand-off cells of every size: 8
+    records (256 owners), 16 (64 owners), 32 (32 owners), 64 (16 owners and fewer), each
+    through the one-launch kernel and through two launches per step."""
+    for N, W, H, auto in ((3000, 64, 64, "persist"), (3000, 32, 32, "persist"), (3000, 32, 16, "two"), (3000, 16, 16, "two"),
+                          (700, 5, 5, "two")):
+        cls, start = gpu.gen_maps_bernoulli(9, 1, N, W, H, 0.12, 0.03)
+        cfg = gpu.make_config(N, W, H, table_mode=gpu.TABLE_SHARED, map_mode=gpu.MAP_SHARED, lr=0.003, eps0=0.3,
+                              episode_len=30, seed=4, trap_reward=-0.5)
+        with gpu.Engine(cfg, 0) as eng:
+            name = eng.fused_kernel_info(50)["name"]
+            assert name == ("k_shared_persist<4,1>" if auto == "persist" else "k_shared_act+k_reduce_owners"), (W, H, name)
+            assert eng.fused_kernel_info(1)["name"] == "k_shared_act+k_reduce_owners"  # too short to repay the set-up
+        for variant in (1, 2):
+            _, q = run_both(gpu, oracle, cfg, cls, start, 40, variant=variant)
+            assert np.isfinite(q).all() and np.count_nonzero(q) > 20
+
+
+@pytest.mark.parametrize("variant", [1, 2])
+def test_shared_table_cells_that_overflow(gpu, oracle, variant):
+    """More distinct keys for one owner than a hand-off cell has records: every env starts
+    (and, with episodes of one step, always acts) on one of the 16 cells that one owner of
+    a 32x32x4 table holds, with random actions - 64 keys for cells of 16 records, in every
+    block and step - so the owners go back to the blocks' raw samples."""
+    N, W, H = 2000, 32, 32
+    cells = np.arange(W * H)
+    hi = cells >> 6                      # 64 owners of 16 cells each
+    owner = (cells + 37 * hi) & 63
+    mine = cells[owner == 5]
+    assert len(mine) == 16
+    rng = np.random.default_rng(3)
+    start = rng.choice(mine, N).astype(np.int32)
+    cls = np.zeros((1, W * H), np.uint8)
+    cfg = gpu.make_config(N, W, H, table_mode=gpu.TABLE_SHARED, map_mode=gpu.MAP_SHARED, lr=0.01, eps0=1.0,
+                          episode_len=1, seed=6)
+    _, q = run_both(gpu, oracle, cfg, cls, start, 30, variant=variant)
+    touched = np.count_nonzero(q.reshape(W * H, 4)[mine])
+    assert touched == 64 and np.count_nonzero(q) == 64
 
 
 def test_shared_table_all_envs_on_one_cell(gpu, oracle):
