@@ -154,12 +154,13 @@ __device__ __forceinline__ void reduce_block_init(ReduceLds& L) {
 // Pass 1 for one block.  All 256 threads of the workgroup call it with their
 // sample (valid = false: no sample / no delta); key < K <= kDenseKeys.  Leaves the
 // LDS state as reduce_block_init() did, so it can be called again and again.
-// The hand-off cell of (block, owner) is 64 bytes at handoff[(block * owners + owner) * 8].
 // DEV = false: the records go straight to memory with plain stores, for a reader in a
-// later launch.
+// later launch; the cell of (owner, block) is at handoff[(owner * blocks + block) << cell_shift],
+// so that an owner reads its cells side by side.
 // DEV = true: for readers on other XCDs in the same launch.  All cells of the block
 // are put together in LDS (`stage`, owners x 8 records, free again on return) and go
-// out as whole lines, 16 bytes to a store and lane, every record carrying `tag`:
+// out as whole lines (the cell of (block, owner) at (block * owners + owner) << cell_shift
+// behind `window_offset`), 16 bytes to a store and lane, every record carrying `tag`:
 // scattered 8-byte stores are partial line writes, and some 350 of them per workgroup
 // took 1.6 us to be acknowledged.  `window` is a buffer window on `handoff`.
 // Returns (to every thread) whether some owner was handed more distinct keys than a
@@ -255,9 +256,9 @@ __device__ __forceinline__ bool reduce_block(ReduceLds& L, const ReduceGeom G, c
         const int c = L.handed[owner];  // final: every leader has drawn its slot
         count = (uint32_t)(c > cap ? kSlotOverflow : c);
       }
-      handoff[((((size_t)block * n_own) + owner) << G.cell_shift) + slot] = make_rec((uint32_t)slot_of(key, G), count, tag, acc);
+      handoff[((((size_t)owner * G.n_blocks) + block) << G.cell_shift) + slot] = make_rec((uint32_t)slot_of(key, G), count, tag, acc);
     }
-    if (tid < n_own && L.handed[tid] == 0) handoff[(((size_t)block * n_own) + tid) << G.cell_shift] = make_rec(0u, 0u, tag, 0.0f);
+    if (tid < n_own && L.handed[tid] == 0) handoff[(((size_t)tid * G.n_blocks) + block) << G.cell_shift] = make_rec(0u, 0u, tag, 0.0f);
   }
   return over;
 }
@@ -300,7 +301,7 @@ __global__ __launch_bounds__(256) void k_reduce_owners(const ReduceGeom G, float
     // the first eight records of the hand-off cell in one go: no load depends on
     // another (a cell with more records has the rest fetched below, when it holds them)
     uint4 cell[kMinCellRecs / 2];
-    const uint4* src = reinterpret_cast<const uint4*>(handoff + ((((size_t)b << G.own_shift) + owner) << G.cell_shift));
+    const uint4* src = reinterpret_cast<const uint4*>(handoff + ((((size_t)owner * G.n_blocks) + b) << G.cell_shift));
     if (b < G.n_blocks) {
 #pragma unroll
       for (int i = 0; i < kMinCellRecs / 2; ++i) cell[i] = src[i];
