@@ -715,6 +715,8 @@ hipError_t launch_persist_kernel(crl_engine* e, const PersistPlan& p, unsigned l
                                     dim3(256), args, (unsigned)p.lds, e->stream);
 }
 
+static_assert(crl::kPersistClockWords == CRL_PERSIST_CLOCK_WORDS, "include/crl.h states the size of the diagnostics");
+
 // -> CRL_OK and *launched = true, or *launched = false when the caller should take
 // the two-launches-per-step path instead
 int run_persist(crl_engine* e, int n_steps, bool* launched) {
@@ -1544,18 +1546,18 @@ int crl_set_persist_clocks(crl_engine* e, int32_t on) {
   return CRL_OK;
 }
 
-// Diagnostics: per-phase shader clocks, summed over the steps of the last one-launch
-// shared-table launch that ran with the clocks armed, of its first (out[0..7]) and
-// last (out[8..15]) workgroup.
-int crl_get_persist_clocks(crl_engine* e, uint64_t* out16) {
+// Diagnostics: what the last one-launch shared-table launch that ran with the clocks armed
+// left behind (layout: include/crl.h); at most n_words 64-bit words are copied.
+int crl_get_persist_clocks(crl_engine* e, uint64_t* out, size_t n_words) {
   int rc = check_engine(e);
   if (rc) return rc;
-  if (!out16) return fail(CRL_E_ARG, "out16 is null");
+  if (!out) return fail(CRL_E_ARG, "out is null");
   if (!e->pdiag.p) return fail(CRL_E_STATE, "this engine has no shared table");
   HIP_TRY(hipStreamSynchronize(e->stream));
   rc = check_persist(e);
   if (rc) return rc;
-  HIP_TRY(hipMemcpy(out16, e->pdiag.p + 1, crl::kPersistClockWords * sizeof(uint64_t), hipMemcpyDeviceToHost));
+  const size_t n = std::min<size_t>(n_words, crl::kPersistClockWords);
+  HIP_TRY(hipMemcpy(out, e->pdiag.p + 1, n * sizeof(uint64_t), hipMemcpyDeviceToHost));
   return CRL_OK;
 }
 

@@ -252,6 +252,10 @@ PYBIND11_MODULE(cudarl_core, m) {
            })
       .def("update", &BatchedEnvironment::update)
       .def("run", &BatchedEnvironment::run, py::arg("n_steps"), py::call_guard<py::gil_scoped_release>())
+      // the same under the name a caller of select / step / update looks for: n fused rounds
+      // in one call instead of 3 n launches (1M envs of 16x16: 1.4e10 env-steps/s one round
+      // per call, 3.1e10 at 20, 8.8e10 at 1000)
+      .def("step_n", &BatchedEnvironment::run, py::arg("n_steps"), py::call_guard<py::gil_scoped_release>())
       .def("sync", &BatchedEnvironment::sync)
       .def("state",
            [](const BatchedEnvironment& self) {

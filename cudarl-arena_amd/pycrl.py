@@ -149,7 +149,7 @@ def load():
     lib.crl_gen_maps_noise.argtypes = [u64, i32, i32, i32, i32, f32, f32, f32, vp, vp, vp]
     lib.crl_probe_copy.argtypes = [C.c_size_t, C.c_int]
     lib.crl_probe_barrier.argtypes = [C.c_int, C.c_int, C.c_int, C.POINTER(C.c_double)]
-    lib.crl_get_persist_clocks.argtypes = [vp, vp]
+    lib.crl_get_persist_clocks.argtypes = [vp, vp, C.c_size_t]
     lib.crl_set_persist_clocks.argtypes = [vp, C.c_int32]
     _lib = lib
     return lib
@@ -385,7 +385,7 @@ class Engine:
         """Per-phase shader clocks of the last one-launch shared-table launch that ran with the
         clocks armed: (first, last workgroup) x 8."""
         out = np.zeros(20 + 8 * 256, np.uint64)
-        _check(self.lib.crl_get_persist_clocks(self.h, _ptr(out)))
+        _check(self.lib.crl_get_persist_clocks(self.h, _ptr(out), out.size))
         self.persist_stamps = out[20:].reshape(256, 8)  # 100 MHz wall clock of every workgroup at the marks of the middle step
         return out[:20].reshape(2, 10)
 

@@ -302,13 +302,20 @@ int crl_probe_copy(size_t n_bytes, int repeats);
 /* Phase clocks of the one-launch shared-table kernel.  crl_set_persist_clocks(e, 1)
  * makes later launches run the instantiation that reads the shader clock between
  * the phases of every step (off by default: the product kernel carries no clocks);
- * crl_get_persist_clocks returns the sums over the steps of the last such launch for
- * its first (out16[0..7]) and last (out16[8..15]) workgroup.  Phases: 0 work that
- * does not need the table, 1 wait for the table, 2 select / move / delta, 3 ordered
- * block sums + cells, 4 clearing the owner's tile, 5 wait for the cells, 6 tile,
- * sums, publish, 7 loop overhead. */
+ * crl_get_persist_clocks copies what the last such launch left, at most n_words
+ * 64-bit words of CRL_PERSIST_CLOCK_WORDS:
+ *   [0..7]   first workgroup: shader clocks per phase, summed over the steps
+ *   [8..9]   first workgroup, thread 0: polls of the table wait / of the cells wait
+ *   [10..19] the same ten words of the last workgroup
+ *   [20 + 8 w + p]  100 MHz wall clock at which workgroup w passed the mark that ends
+ *            phase p in the middle step of the launch (w < 256)
+ * Phases: 0 what a step needs that does not depend on the table, 1 wait for the table,
+ * 2 select / move / delta, 3 ordered block sums + cells, 4 clearing the owner's tile and
+ * waiting for the cells' acknowledgement, 5 wait for the others' cells, 6 tile, sums,
+ * publish, 7 loop overhead. */
+#define CRL_PERSIST_CLOCK_WORDS (20 + 8 * 256)
 int crl_set_persist_clocks(crl_engine* e, int32_t on);
-int crl_get_persist_clocks(crl_engine* e, uint64_t* out16);
+int crl_get_persist_clocks(crl_engine* e, uint64_t* out, size_t n_words);
 /* Nanoseconds per barrier over n_groups (<= 256) co-resident workgroups that meet
  * through device-scope loads and stores.  pattern 0: packed flags, all polled by
  * everybody; 1: one flag per 128-byte line; 2: a tree in which every word has one
