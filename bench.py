@@ -52,7 +52,7 @@ WORKLOADS = {
     # traffic: bytes per env-step past the L2, from rocprofv3 FETCH_SIZE x2.000 + WRITE_SIZE x1.000
     # in separate --pmc runs of the same launches (profiles/*.md), valid for the
     # workload's own launch length only (traffic_short: c4 at 20 steps per launch)
-    "c4": dict(n=1 << 20, launch_steps=1000, bytes=42.25, traffic=29.8, traffic_short={20: 58.1},
+    "c4": dict(n=1 << 20, launch_steps=1000, bytes=42.25, traffic=29.8, traffic_short={20: 58.1, 1: 335.0},
                name="c4: 1048576 envs 16x16, per-env tables 256x4 (4 GB), traps, eps 0.1, T=128, 1000 steps"),
     "c5": dict(n=8192, launch_steps=1024, bytes=70.0, traffic=87.1,
                name="c5: 8192 envs 256x256, 8 actions, per-env tables 65536x8 (16 GB), cell rewards, "
@@ -458,6 +458,9 @@ def main():
             # what a caller that asks for a few steps at a time gets: another launch plan
             # (every env in flight, class maps staged, tables never in LDS)
             also["c4_20_steps_per_launch"] = side_figure("c4", 20, 5, 20)
+            # ... and a caller of one select / step / update round per call: every env's state, map
+            # and table lines come from HBM for a single step (335 B per env-step measured)
+            also["c4_1_step_per_launch"] = side_figure("c4", 40, 5, 1)
         out["also"] = also
     print(json.dumps(out))
 
