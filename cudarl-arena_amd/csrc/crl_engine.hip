@@ -656,7 +656,7 @@ struct PersistPlan {
   size_t lds;
   crl::ReduceGeom G;
   // what the workgroups exchange, in 64-bit words from the start of one buffer
-  size_t at_table, at_rowmax, at_mark, at_raw, at_cells, words;
+  size_t at_table, at_mark, at_raw, at_cells, words;
 };
 
 // Shortest call worth the set-up of the one-launch kernel (clearing what its workgroups
@@ -683,8 +683,7 @@ PersistPlan plan_persist(const crl_engine* e, int n_steps) {
   p.lds = sizeof(crl::PersistLds) + (p.lds_map ? map_bytes : 0);
   auto pad = [](size_t words) { return (words + 31) & ~(size_t)31; };  // 256-byte pieces
   p.at_table = 0;
-  p.at_rowmax = p.at_table + pad(e->K);
-  p.at_mark = p.at_rowmax + pad(e->S);
+  p.at_mark = p.at_table + pad(2 * (size_t)e->K);  // a cell's view: its A values and A neighbours' maxima
   p.at_raw = p.at_mark + pad((size_t)n_own);
   p.at_cells = p.at_raw + pad(2 * (size_t)e->N);  // raw samples and cells: two buffers each
   p.words = p.at_cells + 2 * (((size_t)n_own * p.grid) << p.G.cell_shift);
@@ -701,7 +700,6 @@ hipError_t launch_persist_kernel(crl_engine* e, const PersistPlan& p, unsigned l
   crl::ReduceGeom G = p.G;
   crl::PersistBufs B{};
   B.table = buf + p.at_table;
-  B.rowmax = buf + p.at_rowmax;
   B.mark = buf + p.at_mark;
   B.raw = buf + p.at_raw;
   B.cells = buf + p.at_cells;

@@ -10,22 +10,26 @@
 // are no flags, no "store, wait for the acknowledgement, then publish", and one
 // trip through memory per exchange instead of two.
 //
-//   table[key]   {value, tag}   published by the key's owner
-//   rowmax[cell] {max of the row, tag}   by the owner of the row
+//   view[cell]   2 A units, side by side, everything a step of an env on that cell needs:
+//                  [0, A)   {value, tag} of the cell's A keys, published by the row's owner
+//                  [A, 2A)  {max of the row of the cell that action i leads to, tag},
+//                           published by THAT row's owner (the cell itself where the move
+//                           would leave the grid): one row maximum goes to up to A + 2 places
 //   mark[owner]  {0, tag}       "this owner has consumed the cells of the step before" (read by workgroups that are no owners)
 //   cell[block][owner][8]       block sums, records as in crl_reduce.h; written whole every step
 //   raw[env]     {delta, key, tag}   only from blocks whose cell for some owner overflowed
 //
 // One step k (tag k + 1 for what the blocks read, k + 2 for the table that results):
 //   block:  what does not depend on the table (exploration draw, neighbour cells, move
-//           codes; the owner's stores are on their way meanwhile) -> poll own row and
-//           the A neighbours' row maxima -> select, move, (key, delta) -> ordered block
+//           codes; the owner's stores are on their way meanwhile) -> poll the view of
+//           the env's cell -> select, move, (key, delta) -> ordered block
 //           sums -> cells
 //   owner:  clear the tile, wait until the cells are acknowledged -> poll the cells of
-//           all blocks -> tile -> sums in tree order -> new values, row maxima and mark
+//           all blocks -> tile -> sums in tree order -> new values and row maxima into
+//           the views, mark
 // An owner overwrites its values only after it has every block's cells of the step,
-// which a block writes after all its threads have read theirs: one buffer of table
-// and row maxima suffices.  Cells and raw samples have two buffers, taken in turn: a
+// which a block writes after all its threads have read theirs: one buffer of views
+// suffices.  Cells and raw samples have two buffers, taken in turn: a
 // workgroup that writes the cells of step k + 2 has read table values of step k + 2,
 // so some owner has had the cells of step k + 1 of ALL workgroups, which - a
 // workgroup does its two roles one after the other - were all through with their
@@ -62,8 +66,7 @@ struct alignas(16) PersistLds {
 };
 
 struct PersistBufs {
-  unsigned long long* table;   // [K]
-  unsigned long long* rowmax;  // [S]
+  unsigned long long* table;   // view [S][2 A]
   unsigned long long* mark;    // [owners]
   unsigned long long* cells;   // [owners][workgroups][8]
   unsigned long long* raw;     // [N]
@@ -167,18 +170,31 @@ __global__ __launch_bounds__(256) void k_shared_persist(const Rules R, const Ptr
   const int own_key = key_of(wg, lane, G);
   const bool own_live = is_owner && wave == 0 && own_key < G.K;
   float q_own = own_live ? P.Q[own_key] : 0.0f;
+  // where the lane of action a publishes: its value in the view of its cell, and the row's
+  // maximum in the view of the cell that reaches this one by action a (and in its own
+  // cell's view if action a would leave the grid there)
+  int pub_q = -1, pub_from = -1, pub_self = -1;
+  if (own_live) {
+    const int c = own_key >> G.a_shift, a = own_key & (A - 1);
+    const int x = c % R.W, y = c / R.W;
+    int dx, dy;
+    action_delta(a, A, dx, dy);
+    pub_q = c * 2 * A + a;
+    if ((unsigned)(x - dx) < (unsigned)R.W && (unsigned)(y - dy) < (unsigned)R.H) pub_from = (c - dy * R.W - dx) * 2 * A + A + a;
+    if (!((unsigned)(x + dx) < (unsigned)R.W && (unsigned)(y + dy) < (unsigned)R.H)) pub_self = c * 2 * A + A + a;
+  }
   auto publish = [&](uint32_t tag) {  // wave 0 of an owner
     float qs[A];
 #pragma unroll
     for (int i = 0; i < A; ++i) qs[i] = __shfl(q_own, (lane & ~(A - 1)) + i);
     if (own_live) {
-      st_dev64(B.table + own_key, tagged(__float_as_uint(q_own), tag));
-      if ((lane & (A - 1)) == 0) {
-        Row<A> row;
-        if constexpr (A == 4) row = Row<4>{qs[0], qs[1], qs[2], qs[3]};
-        else row = Row<8>{qs[0], qs[1], qs[2], qs[3], qs[4], qs[5], qs[6], qs[7]};
-        st_dev64(B.rowmax + (own_key >> G.a_shift), tagged(__float_as_uint(row_max(row, false, 0)), tag));
-      }
+      st_dev64(B.table + pub_q, tagged(__float_as_uint(q_own), tag));
+      Row<A> row;
+      if constexpr (A == 4) row = Row<4>{qs[0], qs[1], qs[2], qs[3]};
+      else row = Row<8>{qs[0], qs[1], qs[2], qs[3], qs[4], qs[5], qs[6], qs[7]};
+      const unsigned long long mx = tagged(__float_as_uint(row_max(row, false, 0)), tag);
+      if (pub_from >= 0) st_dev64(B.table + pub_from, mx);
+      if (pub_self >= 0) st_dev64(B.table + pub_self, mx);
     }
     if (lane == 0) st_dev64(B.mark + wg, tagged(0u, tag));
   };
@@ -240,10 +256,10 @@ __global__ __launch_bounds__(256) void k_shared_persist(const Rules R, const Ptr
     CRL_MARK(0);
 
 
-    // ---- the table of this step: own row, the neighbours' maxima, one owner's mark --
+    // ---- the table of this step: the view of the env's cell, one owner's mark ----------
     unsigned long long rq[A], rn[A];
     {
-      const uint32_t qrow = (uint32_t)s0 * (uint32_t)(A * 8);  // byte offset of the row in the table
+      const uint32_t view = (uint32_t)s0 * (uint32_t)(2 * A * 8);  // byte offset of the cell's view
       bool ok = false;
       int spins = 0;
       while (!ok) {
@@ -251,21 +267,19 @@ __global__ __launch_bounds__(256) void k_shared_persist(const Rules R, const Ptr
         unsigned long long mk = tagged(0u, want);
         if (!is_owner && tid < n_own) mk = ld_dev64(B.mark + tid);
         if (live) {
+          // two units to a 16-byte load: the row, then the neighbours' maxima
 #pragma unroll
-          for (int i = 0; i < A; ++i) rn[i] = ld_dev64(B.rowmax + nb[i]);
-          // the row: two values to a 16-byte load
-          const uint4 r0 = ld_dev128(w_table, qrow), r1 = ld_dev128(w_table, qrow + 16);
-          if constexpr (A == 8) {
-            const uint4 r2 = ld_dev128(w_table, qrow + 32), r3 = ld_dev128(w_table, qrow + 48);
-            rq[4] = tagged(r2.x, r2.y);
-            rq[5] = tagged(r2.z, r2.w);
-            rq[6] = tagged(r3.x, r3.y);
-            rq[7] = tagged(r3.z, r3.w);
+          for (int i = 0; i < A; i += 2) {
+            const uint4 r = ld_dev128(w_table, view + (uint32_t)i * 8u);
+            rq[i] = tagged(r.x, r.y);
+            rq[i + 1] = tagged(r.z, r.w);
           }
-          rq[0] = tagged(r0.x, r0.y);
-          rq[1] = tagged(r0.z, r0.w);
-          rq[2] = tagged(r1.x, r1.y);
-          rq[3] = tagged(r1.z, r1.w);
+#pragma unroll
+          for (int i = 0; i < A; i += 2) {
+            const uint4 r = ld_dev128(w_table, view + (uint32_t)(A + i) * 8u);
+            rn[i] = tagged(r.x, r.y);
+            rn[i + 1] = tagged(r.z, r.w);
+          }
         }
         ok = tag_of(mk) == want;
         if (live) {
