@@ -508,6 +508,7 @@ crl::ReduceGeom reduce_geom(const crl_engine* e, int n) {
   G.own_shift = ceil_log2((e->K + crl::kOwnKeys - 1) / crl::kOwnKeys);
   G.n_blocks = (n + crl::kBlockSamples - 1) / crl::kBlockSamples;
   G.cell_shift = crl::cell_shift_for(G.own_shift);
+  G.main_shift = crl::main_shift_for(G.own_shift);
   return G;
 }
 

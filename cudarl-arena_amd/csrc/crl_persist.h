@@ -16,7 +16,8 @@
 //                           published by THAT row's owner (the cell itself where the move
 //                           would leave the grid): one row maximum goes to up to A + 2 places
 //   mark[owner]  {0, tag}       "this owner has consumed the cells of the step before" (read by workgroups that are no owners)
-//   cell[block][owner][8]       block sums, records as in crl_reduce.h; written whole every step
+//   cell[block][owner][records] block sums, records as in crl_reduce.h; its main half written whole
+//                               every step, its extension [owner][block] record by record when needed
 //   raw[env]     {delta, key, tag}   only from blocks whose cell for some owner overflowed
 //
 // One step k (tag k + 1 for what the blocks read, k + 2 for the table that results):
@@ -68,7 +69,7 @@ struct alignas(16) PersistLds {
 struct PersistBufs {
   unsigned long long* table;   // view [S][2 A]
   unsigned long long* mark;    // [owners]
-  unsigned long long* cells;   // [owners][workgroups][8]
+  unsigned long long* cells;   // 2 x [workgroups][owners][main half], then 2 x [owners][workgroups][extension]
   unsigned long long* raw;     // [N]
   unsigned* err;               // give-up word
   unsigned long long* clocks;  // kPersistClockWords phase clocks, or null
@@ -161,7 +162,9 @@ __global__ __launch_bounds__(256) void k_shared_persist(const Rules R, const Ptr
   const uint32_t* gmap = P.map + ((P.map_shared || !has_env) ? 0 : (size_t)env * P.map_words);
   const float* cr = P.cell_reward ? P.cell_reward + ((P.map_shared || !has_env) ? 0 : (size_t)env * P.S) : nullptr;
   const DevWindow w_table = dev_window(B.table), w_cells = dev_window(B.cells);
-  const size_t cells_half = ((size_t)n_own * G.n_blocks) << G.cell_shift;  // 64-bit words of one buffer of cells
+  // 64-bit words of one buffer of main halves; cells with an extension: as many again, behind both buffers
+  const size_t cells_half = ((size_t)n_own * G.n_blocks) << G.main_shift;
+  const bool has_ext = G.main_shift < G.cell_shift;
   const bool cells_flag = (R.reward_flags & 1) != 0;
   const bool base_cells = cells_flag && (R.reward_flags & 2) != 0;
 
@@ -356,7 +359,7 @@ __global__ __launch_bounds__(256) void k_shared_persist(const Rules R, const Ptr
     const int half = k & 1;  // cells and raw samples: two buffers, taken in turn
     const bool over = reduce_block<true>(L.red, G, wg, my_key, my_delta, live, B.cells, want,
                                          reinterpret_cast<unsigned long long*>(L.tile), &w_cells,
-                                         (uint32_t)((size_t)half * cells_half * 8));
+                                         (uint32_t)((size_t)half * cells_half * 8), B.cells + (2 + half) * cells_half);
     if (over && has_env)
       st_dev64(B.raw + (size_t)half * P.N + env, tagged(__float_as_uint(my_delta),
                                    (uint32_t)my_key | (live ? kRawValid : 0u) | (want << kRawTagShift)));
@@ -376,41 +379,54 @@ __global__ __launch_bounds__(256) void k_shared_persist(const Rules R, const Ptr
     // ---- as owner of 64 keys: all blocks' cells, added in tree order --------------------
     if (is_owner) {
       // A wave takes 64 blocks' cells, 16 bytes = two records to a lane and load: the
-      // lanes that share a cell (4 for cells of eight records, up to 32) read it side by
-      // side, so a load of the wave is whole cells instead of 64 pieces of 64 different
-      // ones.  GS loads at a time are asked for, checked and put into the tile: all four
-      // of cells of eight records, eight at a time of larger cells.
+      // lanes that share a cell's main half (2 for halves of four records, up to 32) read
+      // it side by side, so a load of the wave is whole cells instead of 64 pieces of 64
+      // different ones, and the same lanes read the cell's extension.  GS loads of either
+      // at a time are asked for, checked and put into the tile: everything at once for
+      // cells of up to 16 records, eight at a time of larger ones.
       {
-        const int pc_shift = G.cell_shift - 1;            // log2(pieces of a cell)
+        const int pc_shift = G.main_shift - 1;            // log2(pieces of a main half)
         const int pair = lane & ((1 << pc_shift) - 1);    // this lane's piece of its cell
         const int cells_per_load = 64 >> pc_shift;
         const int n_loads = 1 << pc_shift;
-        auto fetch_cells = [&](auto group_size) {
+        const int cap_main = 1 << G.main_shift;
+        auto fetch_cells = [&](auto group_size, auto with_ext) {
           constexpr int GS = decltype(group_size)::value;
+          constexpr bool EXT = decltype(with_ext)::value;
           int spins = 0;
           bool stop = false;
           for (int j0 = 0; j0 < n_loads && !stop; j0 += GS) {
-            uint4 rec[GS];
+            uint4 rec[GS], more[EXT ? GS : 1];
             int cnt[GS];
-            uint32_t src[GS];  // byte offsets into the cells
+            uint32_t src[GS], src_more[EXT ? GS : 1];  // byte offsets into the cells
             bool have[GS];
 #pragma unroll
             for (int j = 0; j < GS; ++j) {
               const int blk = wave * 64 + (j0 + j) * cells_per_load + (lane >> pc_shift);
               have[j] = blk < G.n_blocks;
-              src[j] = (uint32_t)(((size_t)half * cells_half + ((size_t)((have[j] ? blk : 0) * n_own + wg) << G.cell_shift) + 2 * pair) * 8);
+              src[j] = (uint32_t)(((size_t)half * cells_half + ((size_t)((have[j] ? blk : 0) * n_own + wg) << G.main_shift) + 2 * pair) * 8);
+              if (EXT)
+                src_more[j] = (uint32_t)(((size_t)(2 + half) * cells_half + ((size_t)(wg * G.n_blocks + (have[j] ? blk : 0)) << G.main_shift) + 2 * pair) * 8);
             }
             for (;;) {
               poll_fence();
 #pragma unroll
               for (int j = 0; j < GS; ++j) rec[j] = ld_dev128(w_cells, src[j]);
+              if (EXT) {
+#pragma unroll
+                for (int j = 0; j < GS; ++j) more[j] = ld_dev128(w_cells, src_more[j]);
+              }
               bool ok = true;
 #pragma unroll
               for (int j = 0; j < GS; ++j) {
                 const uint32_t meta0 = (uint32_t)__shfl((int)rec[j].x, lane - pair);
                 cnt[j] = rec_count(meta0);
-                // (every record of a cell is written every step)
-                const bool mine = rec_tag(meta0) == want && rec_tag(rec[j].x) == want && rec_tag(rec[j].z) == want;
+                // (every record of a main half is written every step)
+                bool mine = rec_tag(meta0) == want && rec_tag(rec[j].x) == want && rec_tag(rec[j].z) == want;
+                if (EXT && cnt[j] != kSlotOverflow) {  // (an extension record: only where the count says so)
+                  mine = mine && (cap_main + 2 * pair >= cnt[j] || rec_tag(more[j].x) == want) &&
+                         (cap_main + 2 * pair + 1 >= cnt[j] || rec_tag(more[j].z) == want);
+                }
                 ok = ok && (mine || !have[j]);
               }
               if (__all(ok)) break;
@@ -436,13 +452,18 @@ __global__ __launch_bounds__(256) void k_shared_persist(const Rules R, const Ptr
                 } else {
                   if (2 * pair < cnt[j]) row[rec_slot(rec[j].x)] = __uint_as_float(rec[j].y);
                   if (2 * pair + 1 < cnt[j]) row[rec_slot(rec[j].z)] = __uint_as_float(rec[j].w);
+                  if (EXT) {
+                    if (cap_main + 2 * pair < cnt[j]) row[rec_slot(more[j].x)] = __uint_as_float(more[j].y);
+                    if (cap_main + 2 * pair + 1 < cnt[j]) row[rec_slot(more[j].z)] = __uint_as_float(more[j].w);
+                  }
                 }
               }
             }
           }
         };
-        if (n_loads == 4) fetch_cells(std::integral_constant<int, 4>{});
-        else fetch_cells(std::integral_constant<int, 8>{});
+        if (has_ext && n_loads == 2) fetch_cells(std::integral_constant<int, 2>{}, std::true_type{});
+        else if (has_ext && n_loads == 4) fetch_cells(std::integral_constant<int, 4>{}, std::true_type{});
+        else fetch_cells(std::integral_constant<int, 8>{}, std::false_type{});
       }
       CRL_MARK(5);
       __syncthreads();

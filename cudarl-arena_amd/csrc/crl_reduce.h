@@ -56,6 +56,7 @@ struct ReduceGeom {
   int own_shift;  // log2(number of owners); owners = 1 << own_shift, (K >> own_shift) <= 64
   int n_blocks;   // ceil(n / 256)
   int cell_shift; // log2(records of a hand-off cell), cell_shift_for(own_shift)
+  int main_shift; // one-launch kernel: log2(records in the part of a cell that is written every step), main_shift_for()
 };
 
 // Records per hand-off cell.  A block's 256 samples spread over the owners, so a cell
@@ -65,6 +66,20 @@ struct ReduceGeom {
 // cells together stay within 16 KB.
 __host__ __device__ constexpr int cell_shift_for(int own_shift) {
   return own_shift >= 8 ? 3 : own_shift >= 6 ? 4 : own_shift == 5 ? 5 : 6;
+}
+
+// One-launch kernel: what a block's cell stores cost grows with their bytes (16 KB of
+// cells of eight records for 256 owners, seven eighths of them padding, need 1.4 us to be
+// acknowledged, 8 KB half of that).  So with more than 64 owners a cell is two halves:
+// the main half, written whole every step with all the others of the block (8 KB), and
+// an extension of as many records that only a block with more distinct keys for that
+// owner than the main half holds writes into (one cell in 270 with 256 owners), record by
+// record.  Record 0 of the main half says how many records there are in all.  The
+// extensions lie [owner][block]: an owner asks for all of them with its main halves,
+// 8 KB in one piece, and looks at those the counts point to.
+__host__ __device__ constexpr int main_shift_for(int own_shift) {
+  const int c = cell_shift_for(own_shift), m = 10 - own_shift;
+  return m < c ? (m < 2 ? 2 : m) : c;
 }
 
 // key <-> (owner, slot in the owner's 64).  An owner holds whole table rows:
@@ -158,9 +173,11 @@ __device__ __forceinline__ void reduce_block_init(ReduceLds& L) {
 // later launch; the cell of (owner, block) is at handoff[(owner * blocks + block) << cell_shift],
 // so that an owner reads its cells side by side.
 // DEV = true: for readers on other XCDs in the same launch.  All cells of the block
-// are put together in LDS (`stage`, owners x 8 records, free again on return) and go
-// out as whole lines (the cell of (block, owner) at (block * owners + owner) << cell_shift
-// behind `window_offset`), 16 bytes to a store and lane, every record carrying `tag`:
+// main halves are put together in LDS (`stage`, owners << main_shift records, free again
+// on return) and go out as whole lines (that of (block, owner) at (block * owners + owner)
+// << main_shift behind `window_offset`), 16 bytes to a store and lane, every record
+// carrying `tag`; a record beyond the main half goes straight to
+// ext[(owner * blocks + block) << main_shift]:
 // scattered 8-byte stores are partial line writes, and some 350 of them per workgroup
 // took 1.6 us to be acknowledged.  `window` is a buffer window on `handoff`.
 // Returns (to every thread) whether some owner was handed more distinct keys than a
@@ -173,7 +190,7 @@ __device__ __forceinline__ void reduce_block_init(ReduceLds& L) {
 __device__ __forceinline__ void reduce_stage_init(unsigned long long* stage, const ReduceGeom G, const uint32_t tag) {
   const unsigned long long none = make_rec(0u, 0u, tag, 0.0f);
   ulonglong2* stage2 = reinterpret_cast<ulonglong2*>(stage);
-  for (int i = threadIdx.x; i < 1 << (G.cell_shift - 1 + G.own_shift); i += kBlockSamples) stage2[i] = make_ulonglong2(none, none);
+  for (int i = threadIdx.x; i < 1 << (G.main_shift - 1 + G.own_shift); i += kBlockSamples) stage2[i] = make_ulonglong2(none, none);
 }
 
 template <bool DEV>
@@ -181,10 +198,11 @@ __device__ __forceinline__ bool reduce_block(ReduceLds& L, const ReduceGeom G, c
                                              const int key, const float delta, const bool valid,
                                              unsigned long long* handoff, const uint32_t tag,
                                              unsigned long long* stage = nullptr, const DevWindow* window = nullptr,
-                                             const uint32_t window_offset = 0) {
+                                             const uint32_t window_offset = 0, unsigned long long* ext = nullptr) {
   const int tid = threadIdx.x;
   const int n_own = 1 << G.own_shift;
   const int cap = 1 << G.cell_shift;  // records of a cell
+  const int cap_main = 1 << G.main_shift;  // DEV: of its main half
   if (valid) atomicMin(&L.lead[key], (uint32_t)tid);
   L.delta[tid] = delta;
   __syncthreads();
@@ -222,7 +240,11 @@ __device__ __forceinline__ bool reduce_block(ReduceLds& L, const ReduceGeom G, c
     slot = atomicAdd(&L.handed[owner], 1);  // slot order is free: records carry the key
     if (slot >= cap) L.over = 1;
     // (record 0's count is added on the way out, when every leader has drawn its slot)
-    if (DEV && slot < cap) stage[(owner << G.cell_shift) + slot] = make_rec((uint32_t)slot_of(key, G), 0u, tag, acc);
+    if (DEV && slot < cap) {
+      const unsigned long long rec = make_rec((uint32_t)slot_of(key, G), 0u, tag, acc);
+      if (slot < cap_main) stage[(owner << G.main_shift) + slot] = rec;
+      else st_dev64(ext + ((((size_t)owner * G.n_blocks + block) << G.main_shift) + (slot - cap_main)), rec);
+    }
   }
   __syncthreads();
   const bool over = L.over != 0;
@@ -230,7 +252,7 @@ __device__ __forceinline__ bool reduce_block(ReduceLds& L, const ReduceGeom G, c
   if (DEV) {
     // (at most kStagePieces pieces = four to a thread, all asked for before the first is used)
     const ulonglong2* stage2 = reinterpret_cast<const ulonglong2*>(stage);
-    const int piece_shift = G.cell_shift - 1;  // log2(pieces of a cell)
+    const int piece_shift = G.main_shift - 1;  // log2(pieces of a cell's main half)
     const int pieces = n_own << piece_shift;
     constexpr int kPer = kStagePieces / kBlockSamples;
     ulonglong2 v[kPer];
@@ -246,7 +268,7 @@ __device__ __forceinline__ bool reduce_block(ReduceLds& L, const ReduceGeom G, c
       const int i = tid + j * kBlockSamples;
       v[j].x |= (unsigned long long)(uint32_t)(c[j] > cap ? kSlotOverflow : c[j]) << kRecCountShift;
       if (i < pieces)
-        st_dev128(*window, window_offset + (uint32_t)((((size_t)block * n_own) << (G.cell_shift + 3)) + (size_t)i * 16),
+        st_dev128(*window, window_offset + (uint32_t)((((size_t)block * n_own) << (G.main_shift + 3)) + (size_t)i * 16),
                   make_uint4((uint32_t)v[j].x, (uint32_t)(v[j].x >> 32), (uint32_t)v[j].y, (uint32_t)(v[j].y >> 32)));
     }
   } else {
