@@ -534,7 +534,7 @@ hipError_t allow_lds(Kern kern, size_t bytes) {
 int opt_in_lds(crl_engine* e) {
   if (e->lds_opt_in) return CRL_OK;
   const size_t act = kLdsPerWorkgroup;  // what a launch asks for is checked against this
-  HIP_TRY(allow_lds(crl::k_reduce_blocks, sizeof(crl::ReduceLds)));
+  HIP_TRY(allow_lds(crl::k_reduce_blocks, crl::kReduceLdsBytes));
   HIP_TRY(allow_lds(crl::k_reduce_owners, kOwnersLds));
   HIP_TRY(allow_lds(crl::k_shared_act<4, 1, true>, act - kStaticLdsReserve));
   HIP_TRY(allow_lds(crl::k_shared_act<4, 2, true>, act - kStaticLdsReserve));
@@ -595,7 +595,7 @@ int reduce_apply(crl_engine* e, float* Q, const int32_t* key, const float* delta
   int rc = ensure_handoff(e, G);
   if (rc) return rc;
   hipLaunchKernelGGL(crl::k_reduce_blocks, dim3(G.n_blocks), dim3(crl::kBlockSamples),
-                     sizeof(crl::ReduceLds), e->stream, G, key, delta, n, e->ho);
+                     crl::kReduceLdsBytes, e->stream, G, key, delta, n, e->ho);
   HIP_TRY(hipGetLastError());
   return reduce_owners(e, G, Q, key, delta, n);
 }
@@ -605,7 +605,7 @@ void launch_shared_act(crl_engine* e, bool reduce, const crl::ReduceGeom& G, uin
   const crl::Rules R = e->rules();
   const crl::Ptrs P = e->ptrs();
   const int block = 256, grid = (e->N + block - 1) / block;
-  const size_t lds = (reduce ? sizeof(crl::ReduceLds) : 0) + (MAP == 1 ? (size_t)e->map_words * 4 : 0);
+  const size_t lds = (reduce ? crl::kReduceLdsBytes : 0) + (MAP == 1 ? (size_t)e->map_words * 4 : 0);
   if (reduce)
     hipLaunchKernelGGL((crl::k_shared_act<A, MAP, true>), dim3(grid), dim3(block), lds, e->stream, R, P,
                        t, trace_row, e->key.p, e->delta.p, G, e->ho);
@@ -626,7 +626,7 @@ int shared_step(crl_engine* e, uint64_t t, int trace_row) {
   // shared table itself stays in L2: streaming its 64 KB into every workgroup's
   // LDS each step measured slower than the row reads it saves (12.4 against 12.05 us
   // per step on 65,536 envs, also against the five speculative reads per env).
-  size_t lds = fast ? sizeof(crl::ReduceLds) : 0;
+  size_t lds = fast ? crl::kReduceLdsBytes : 0;
   const size_t limit = fast ? kLdsPerWorkgroup - kStaticLdsReserve : (size_t)64 * 1024;
   const size_t map_bytes = (size_t)e->map_words * 4;
   const bool lds_map = e->cfg.map_mode == CRL_MAP_SHARED && map_bytes <= (size_t)kLdsMapLimitBytes &&

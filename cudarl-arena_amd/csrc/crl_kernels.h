@@ -893,7 +893,7 @@ __global__ __launch_bounds__(256) void k_shared_act(const Rules R, const Ptrs P,
                                                      float* __restrict__ delta, const ReduceGeom G,
                                                      unsigned long long* __restrict__ handoff) {
   extern __shared__ __align__(16) unsigned char lds_raw[];
-  uint32_t* lds_map = reinterpret_cast<uint32_t*>(lds_raw + (REDUCE ? sizeof(ReduceLds) : 0));
+  uint32_t* lds_map = reinterpret_cast<uint32_t*>(lds_raw + (REDUCE ? kReduceLdsBytes : 0));
   const int tid = threadIdx.x;
   const int env = blockIdx.x * blockDim.x + tid;
   bool live = env < P.N;
@@ -989,7 +989,7 @@ __global__ __launch_bounds__(256) void k_shared_act(const Rules R, const Ptrs P,
   }
   if (REDUCE) {
     ReduceLds& L = *reinterpret_cast<ReduceLds*>(lds_raw);
-    reduce_block<false>(L, G, blockIdx.x, my_key, my_delta, live, handoff, 0u);
+    reduce_block<false>(L, G, blockIdx.x, my_key, my_delta, live, handoff, 0u, reinterpret_cast<float*>(lds_raw + sizeof(ReduceLds)));
   }
 }
 

@@ -126,6 +126,7 @@ __global__ __launch_bounds__(256) void k_shared_persist(const Rules R, const Ptr
   extern __shared__ __align__(16) unsigned char lds_raw[];
   PersistLds& L = *reinterpret_cast<PersistLds*>(lds_raw);
   static_assert(sizeof(PersistLds) % 16 == 0 && offsetof(PersistLds, tile) % 16 == 0, "16-byte LDS accesses");
+  static_assert(kStagePieces * 16 + kSortBytes <= sizeof(L.tile), "cell staging and the holders' line-up share the tile");
   uint32_t* lds_map = reinterpret_cast<uint32_t*>(lds_raw + sizeof(PersistLds));
   const int tid = threadIdx.x;
   const int lane = tid & 63;
@@ -357,7 +358,8 @@ __global__ __launch_bounds__(256) void k_shared_persist(const Rules R, const Ptr
 
     // ---- block sums to the owners' cells ------------------------------------------------
     const int half = k & 1;  // cells and raw samples: two buffers, taken in turn
-    const bool over = reduce_block<true>(L.red, G, wg, my_key, my_delta, live, B.cells, want,
+    // (`sorted`: the upper half of the tile; the staging area of the cells is in its first 8 KB)
+    const bool over = reduce_block<true>(L.red, G, wg, my_key, my_delta, live, B.cells, want, L.tile + kTileBlocks * kOwnKeys / 2,
                                          reinterpret_cast<unsigned long long*>(L.tile), &w_cells,
                                          (uint32_t)((size_t)half * cells_half * 8), B.cells + (2 + half) * cells_half);
     if (over && has_env)

@@ -154,6 +154,12 @@ struct alignas(16) ReduceLds {  // (lead and members are also accessed 16 bytes 
   int over;                                      // some owner was handed more than a cell holds
 };
 
+// Besides ReduceLds, reduce_block() needs kSortBytes of LDS for `sorted`: the deltas of a
+// key's further holders, lined up for its leader ([place among the holders][leader]).
+constexpr int kSortRows = 32;
+constexpr size_t kSortBytes = (size_t)kSortRows * kBlockSamples * sizeof(float);
+constexpr size_t kReduceLdsBytes = sizeof(ReduceLds) + kSortBytes;  // ReduceLds, then `sorted`
+
 // Once per kernel, before the first reduce_block() and separated from it by a barrier.
 __device__ __forceinline__ void reduce_block_init(ReduceLds& L) {
   const int tid = threadIdx.x;
@@ -196,7 +202,7 @@ __device__ __forceinline__ void reduce_stage_init(unsigned long long* stage, con
 template <bool DEV>
 __device__ __forceinline__ bool reduce_block(ReduceLds& L, const ReduceGeom G, const int block,
                                              const int key, const float delta, const bool valid,
-                                             unsigned long long* handoff, const uint32_t tag,
+                                             unsigned long long* handoff, const uint32_t tag, float* sorted,
                                              unsigned long long* stage = nullptr, const DevWindow* window = nullptr,
                                              const uint32_t window_offset = 0, unsigned long long* ext = nullptr) {
   const int tid = threadIdx.x;
@@ -214,24 +220,60 @@ __device__ __forceinline__ bool reduce_block(ReduceLds& L, const ReduceGeom G, c
     if (ld != (uint32_t)tid) atomicOr(&L.members[ld][tid >> 6], 1ull << (tid & 63));
   }
   __syncthreads();
+  // A key's sum is its samples' deltas added in thread order, one after the other: the
+  // leader has to walk through them.  Every further holder finds its place among them
+  // (the set bits below its own) and puts its delta there, all at once, so that the
+  // leader's walk is loads from known addresses, several in flight, instead of one bit
+  // scan, load and add after the other (envs that crowd on a few cells: 14 holders of
+  // one key in most blocks, 1 us of such a walk).
   const bool leader = valid && ld == (uint32_t)tid;
+  unsigned long long mw[4] = {0ull, 0ull, 0ull, 0ull};
+  int holders = 0;  // leader: the key's further holders
+  if (valid) {
+    const ulonglong2 lo = *reinterpret_cast<const ulonglong2*>(&L.members[ld][0]);
+    const ulonglong2 hi = *reinterpret_cast<const ulonglong2*>(&L.members[ld][2]);
+    mw[0] = lo.x;
+    mw[1] = lo.y;
+    mw[2] = hi.x;
+    mw[3] = hi.y;
+    const int p0 = __popcll(mw[0]), p1 = __popcll(mw[1]), p2 = __popcll(mw[2]), p3 = __popcll(mw[3]);
+    if (leader) {
+      holders = p0 + p1 + p2 + p3;
+    } else {
+      const int w = tid >> 6;
+      const unsigned long long mine = w == 0 ? mw[0] : w == 1 ? mw[1] : w == 2 ? mw[2] : mw[3];
+      const int place = (w > 0 ? p0 : 0) + (w > 1 ? p1 : 0) + (w > 2 ? p2 : 0) + __popcll(mine & ((1ull << (tid & 63)) - 1ull));
+      if (place < kSortRows) sorted[place * kBlockSamples + (int)ld] = delta;
+    }
+  }
+  __syncthreads();
   float acc = 0.0f;
   int slot = 0, owner = 0;
   if (leader) {
     acc = acc + delta;  // the leader is the key's first sample; the other holders come after it
-    const ulonglong2 lo = *reinterpret_cast<const ulonglong2*>(&L.members[tid][0]);
-    const ulonglong2 hi = *reinterpret_cast<const ulonglong2*>(&L.members[tid][2]);
-    unsigned long long mw[4] = {lo.x, lo.y, hi.x, hi.y};
-    if ((mw[0] | mw[1] | mw[2] | mw[3]) != 0ull) {
+    if (holders != 0) {
       *reinterpret_cast<ulonglong2*>(&L.members[tid][0]) = make_ulonglong2(0ull, 0ull);
       *reinterpret_cast<ulonglong2*>(&L.members[tid][2]) = make_ulonglong2(0ull, 0ull);
+      const int lined = holders < kSortRows ? holders : kSortRows;
+      for (int r0 = 0; r0 < lined; r0 += 4) {
+        float d[4];
 #pragma unroll
-      for (int w = 0; w < 4; ++w) {
-        unsigned long long m = mw[w];
-        while (m != 0ull) {
-          const int j = __builtin_ctzll(m);
-          acc = acc + L.delta[w * 64 + j];  // thread order = sample order
-          m &= m - 1ull;
+        for (int i = 0; i < 4; ++i) d[i] = sorted[(r0 + i < kSortRows ? r0 + i : kSortRows - 1) * kBlockSamples + tid];
+#pragma unroll
+        for (int i = 0; i < 4; ++i)
+          if (r0 + i < lined) acc = acc + d[i];  // thread order = sample order
+      }
+      if (holders > kSortRows) {  // more holders than places: the rest one by one
+        int seen = 0;
+#pragma unroll
+        for (int w = 0; w < 4; ++w) {
+          unsigned long long m = mw[w];
+          while (m != 0ull) {
+            const int j = __builtin_ctzll(m);
+            if (seen >= kSortRows) acc = acc + L.delta[w * 64 + j];
+            ++seen;
+            m &= m - 1ull;
+          }
         }
       }
     }
@@ -299,7 +341,7 @@ __global__ __launch_bounds__(kBlockSamples) void k_reduce_blocks(const ReduceGeo
   const bool valid = k >= 0;
   const float d = valid ? delta[i] : 0.0f;
   __syncthreads();
-  reduce_block<false>(L, G, blockIdx.x, valid ? k : 0, d, valid, handoff, 0u);
+  reduce_block<false>(L, G, blockIdx.x, valid ? k : 0, d, valid, handoff, 0u, reinterpret_cast<float*>(lds_raw + sizeof(ReduceLds)));
 }
 
 // Pass 2: one workgroup per owner (64 keys).
