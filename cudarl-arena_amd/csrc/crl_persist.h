@@ -25,7 +25,7 @@
 //           codes; the owner's stores are on their way meanwhile) -> poll the view of
 //           the env's cell -> select, move, (key, delta) -> ordered block
 //           sums -> cells
-//   owner:  clear the tile, wait until the cells are acknowledged -> poll the cells of
+//   owner:  clear the tile, a short pause -> poll the cells of
 //           all blocks -> tile -> sums in tree order -> new values and row maxima into
 //           the views, mark
 // An owner overwrites its values only after it has every block's cells of the step,
@@ -51,7 +51,8 @@ namespace crl {
 constexpr int kPersistSpinLimit = 1 << 20;  // polls of a fraction of a microsecond each
 constexpr int kPersistMaxGroups = 256;      // workgroups: one per compute unit, all resident
 constexpr int kPersistMaxSteps = 65535;     // per launch: the raw samples' tags have 17 bits
-constexpr int kPersistTablePause = 4;       // x 128 clocks between a step's preparation and its first look at the table
+constexpr int kPersistTablePause = 2;       // x 128 clocks between a step's preparation and its first look at the table
+constexpr int kPersistCellsPause = 4;       // x 128 clocks between clearing the tile and the first look at the cells
 constexpr int kPersistClockWords = 20 + 8 * 256;  // 2 workgroups x (8 phases + polls of the two waits by thread 0),
                                                   // then the wall clock of every workgroup at the 8 marks of one step
 
@@ -255,7 +256,7 @@ __global__ __launch_bounds__(256) void k_shared_persist(const Rules R, const Ptr
     // A first look that comes too early costs a whole round trip more than one that comes
     // just in time: the values published at the end of the last step need about 1.5 us to
     // be visible, the preparation above takes 1 us (65,536 envs on 64x64x4, us per step by
-    // pause: none 8.16, 4 x 128 clocks 7.78, 6 x 7.85, 8 x 7.91, 16 x 8.55).
+    // pause: none 7.10, 2 x 128 clocks 6.98, 4 x 7.04, 6 x 7.14, 8 x 7.24).
     for (int i = 0; i < kPersistTablePause; ++i) __builtin_amdgcn_s_sleep(2);
     CRL_MARK(0);
 
@@ -373,9 +374,10 @@ __global__ __launch_bounds__(256) void k_shared_persist(const Rules R, const Ptr
 #pragma unroll
       for (int i = 0; i < kTileBlocks * kOwnKeys / 4 / 256; ++i) tile4[i * 256 + tid] = make_float4(0.0f, 0.0f, 0.0f, 0.0f);
     }
-    // the cells are acknowledged before the first look at the others': asking while
-    // stores are still on their way takes longer than waiting for them (measured)
-    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    // A short pause before the first look at the others' cells: asking while the own
+    // stores have only just left takes longer (no pause 7.06 us per step, 4 x 128 clocks
+    // 6.97, 8 x 7.03, 12 x 7.56; waiting until the 8 KB of own cells are acknowledged 7.30).
+    for (int i = 0; i < kPersistCellsPause; ++i) __builtin_amdgcn_s_sleep(2);
     CRL_MARK(4);
 
     // ---- as owner of 64 keys: all blocks' cells, added in tree order --------------------
