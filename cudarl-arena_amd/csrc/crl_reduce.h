@@ -282,14 +282,14 @@ __device__ __forceinline__ bool reduce_block(ReduceLds& L, const ReduceGeom G, c
     slot = atomicAdd(&L.handed[owner], 1);  // slot order is free: records carry the key
     if (slot >= cap) L.over = 1;
     // (record 0's count is added on the way out, when every leader has drawn its slot)
-    if (DEV && slot < cap) {
-      const unsigned long long rec = make_rec((uint32_t)slot_of(key, G), 0u, tag, acc);
-      if (slot < cap_main) stage[(owner << G.main_shift) + slot] = rec;
-      else st_dev64(ext + ((((size_t)owner * G.n_blocks + block) << G.main_shift) + (slot - cap_main)), rec);
-    }
+    if (DEV && slot < cap_main) stage[(owner << G.main_shift) + slot] = make_rec((uint32_t)slot_of(key, G), 0u, tag, acc);
   }
   __syncthreads();
   const bool over = L.over != 0;
+  // (behind the barrier: a barrier waits for the stores before it to be acknowledged)
+  if (DEV && leader && slot >= cap_main && slot < cap)
+    st_dev64(ext + ((((size_t)owner * G.n_blocks + block) << G.main_shift) + (slot - cap_main)),
+             make_rec((uint32_t)slot_of(key, G), 0u, tag, acc));
 
   if (DEV) {
     // (at most kStagePieces pieces = four to a thread, all asked for before the first is used)
