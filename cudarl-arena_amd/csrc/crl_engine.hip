@@ -657,7 +657,7 @@ struct PersistPlan {
   size_t lds;
   crl::ReduceGeom G;
   // what the workgroups exchange, in 64-bit words from the start of one buffer
-  size_t at_table, at_mark, at_raw, at_cells, words;
+  size_t at_table, at_raw, at_cells, words;
 };
 
 // Shortest call worth the set-up of the one-launch kernel (clearing what its workgroups
@@ -671,21 +671,22 @@ PersistPlan plan_persist(const crl_engine* e, int n_steps) {
   if (e->cfg.table_mode != CRL_TABLE_SHARED || e->fused_variant == 1 || e->persist_refused) return p;
   if (e->fused_variant == 0 && n_steps < kPersistMinSteps) return p;
   const int n_blocks = (e->N + crl::kBlockSamples - 1) / crl::kBlockSamples;
+  if (e->K > (size_t)crl::kDenseKeys || n_blocks > crl::kPersistMaxGroups || crl::kPersistMaxGroups > kComputeUnits) return p;
+  // always 256 workgroups, each a block (with or without envs) and an owner (with or
+  // without keys): 16,384 keys at most are 64 to an owner
   p.G = reduce_geom(e, e->N);
-  const int n_own = 1 << p.G.own_shift;
-  p.grid = std::max(n_blocks, n_own);
-  if (e->K > (size_t)crl::kDenseKeys || p.grid > crl::kPersistMaxGroups || p.grid > kComputeUnits) return p;
-  // (few owners have large hand-off cells, fetched eight loads at a time; 65,536 envs on a
-  // 16x16x4 table: 14.5 us per step in one launch, 10.3 with two launches per step)
-  if (e->fused_variant == 0 && p.G.cell_shift > 4) return p;
+  p.G.own_shift = crl::kPersistOwnShift;
+  p.G.cell_shift = crl::cell_shift_for(p.G.own_shift);
+  p.G.main_shift = crl::main_shift_for(p.G.own_shift);
+  p.grid = crl::kPersistMaxGroups;
   p.G.n_blocks = p.grid;  // workgroups without envs hand over empty cells
+  const int n_own = 1 << p.G.own_shift;
   const size_t map_bytes = (size_t)e->map_words * 4;
   p.lds_map = e->cfg.map_mode == CRL_MAP_SHARED && sizeof(crl::PersistLds) + map_bytes <= kLdsPerWorkgroup - kStaticLdsReserve;
   p.lds = sizeof(crl::PersistLds) + (p.lds_map ? map_bytes : 0);
   auto pad = [](size_t words) { return (words + 31) & ~(size_t)31; };  // 256-byte pieces
   p.at_table = 0;
-  p.at_mark = p.at_table + pad(2 * (size_t)e->K);  // a cell's view: its A values and A neighbours' maxima
-  p.at_raw = p.at_mark + pad((size_t)n_own);
+  p.at_raw = p.at_table + pad(2 * (size_t)e->K);  // a cell's view: its A values and A neighbours' maxima
   p.at_cells = p.at_raw + pad(2 * (size_t)e->N);  // raw samples and cells: two buffers each
   p.words = p.at_cells + 2 * (((size_t)n_own * p.grid) << p.G.cell_shift);
   if (e->no_alloc && p.words * sizeof(unsigned long long) > kScratchExchangeBytes) return p;
@@ -701,7 +702,6 @@ hipError_t launch_persist_kernel(crl_engine* e, const PersistPlan& p, unsigned l
   crl::ReduceGeom G = p.G;
   crl::PersistBufs B{};
   B.table = buf + p.at_table;
-  B.mark = buf + p.at_mark;
   B.raw = buf + p.at_raw;
   B.cells = buf + p.at_cells;
   B.err = reinterpret_cast<unsigned*>(e->pdiag.p);

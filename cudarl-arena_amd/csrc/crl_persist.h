@@ -1,7 +1,12 @@
-// Shared table, all steps of a launch in ONE kernel: every workgroup is a block of
-// the ordered reduction (256 envs, state in registers for the whole launch) and
-// the owner of 64 keys (64 / A whole table rows, values in registers), and the two
-// roles hand their data to each other through memory.
+// Shared table, all steps of a launch in ONE kernel: 256 workgroups, one per compute
+// unit, every one of them a block of the ordered reduction (256 envs, state in
+// registers for the whole launch; fewer envs: blocks without envs) and the owner of up
+// to 64 keys (whole table rows, values in registers), and the two roles hand their
+// data to each other through memory.  Always 256 owners, also where the table would
+// fit fewer: an owner's 256 cells are then small ones, every workgroup has a part in
+// both passes, and a table of few cells that many envs crowd on is spread as far as
+// it goes (65,536 envs on a 16x16x4 table: 7.2 us per step with 256 owners of one row
+// each, 14.3 with 16 owners of 16 rows).
 //
 // What is exchanged is only ever touched with device-scope accesses (st_dev64 /
 // ld_dev64: coherent between the eight XCDs without fences), and every exchanged
@@ -15,29 +20,26 @@
 //                  [A, 2A)  {max of the row of the cell that action i leads to, tag},
 //                           published by THAT row's owner (the cell itself where the move
 //                           would leave the grid): one row maximum goes to up to A + 2 places
-//   mark[owner]  {0, tag}       "this owner has consumed the cells of the step before" (read by workgroups that are no owners)
-//   cell[block][owner][records] block sums, records as in crl_reduce.h; its main half written whole
-//                               every step, its extension [owner][block] record by record when needed
+//   cell[block][owner]          block sums, records as in crl_reduce.h: a main half of 4 records,
+//                               written whole every step ([block][owner]: 8 KB of whole lines per
+//                               block), and an extension of 4 more ([owner][block]) that only a
+//                               block with more than 4 distinct keys for that owner writes into
 //   raw[env]     {delta, key, tag}   only from blocks whose cell for some owner overflowed
 //
 // One step k (tag k + 1 for what the blocks read, k + 2 for the table that results):
 //   block:  what does not depend on the table (exploration draw, neighbour cells, move
 //           codes; the owner's stores are on their way meanwhile) -> poll the view of
-//           the env's cell -> select, move, (key, delta) -> ordered block
-//           sums -> cells
-//   owner:  clear the tile, a short pause -> poll the cells of
-//           all blocks -> tile -> sums in tree order -> new values and row maxima into
-//           the views, mark
+//           the env's cell -> select, move, (key, delta) -> ordered block sums -> cells
+//   owner:  clear the tile, a short pause -> poll the cells of all blocks -> tile ->
+//           sums in tree order -> new values and row maxima into the views
 // An owner overwrites its values only after it has every block's cells of the step,
 // which a block writes after all its threads have read theirs: one buffer of views
-// suffices.  Cells and raw samples have two buffers, taken in turn: a
-// workgroup that writes the cells of step k + 2 has read table values of step k + 2,
-// so some owner has had the cells of step k + 1 of ALL workgroups, which - a
-// workgroup does its two roles one after the other - were all through with their
-// owner's part of step k by then.  That argument needs a workgroup to wait for table
-// values or, as an owner, for cells; a workgroup that is no owner (more blocks than
-// owners) might have no env left to wait for, so those poll every owner's mark
-// (one thread each) as well.
+// suffices.  Cells and raw samples have two buffers, taken in turn: a workgroup that
+// writes the cells of step k + 2 has read table values of step k + 2 (or, without
+// envs, has had all cells of step k + 1 as an owner), so some owner has had the
+// cells of step k + 1 of ALL workgroups, which - a workgroup does its two roles one
+// after the other, and every workgroup writes cells every step, empty ones if it has
+// no envs - were all through with their owner's part of step k by then.
 //
 // Every wait is bounded: a thread that polls `spin_limit` times in vain (or sees the
 // give-up word set) makes its workgroup set the give-up word and leave.
@@ -50,6 +52,10 @@ namespace crl {
 
 constexpr int kPersistSpinLimit = 1 << 20;  // polls of a fraction of a microsecond each
 constexpr int kPersistMaxGroups = 256;      // workgroups: one per compute unit, all resident
+constexpr int kPersistOwnShift = 8;         // log2(owners): always 256, every workgroup is one
+constexpr int kMainShift = 2, kMainRecs = 1 << kMainShift;  // records in the half of a cell that is written every step
+static_assert(main_shift_for(kPersistOwnShift) == kMainShift && cell_shift_for(kPersistOwnShift) == kMainShift + 1 &&
+              (1 << kPersistOwnShift) == kPersistMaxGroups, "the owner's loads are laid out for cells of 4 + 4 records");
 constexpr int kPersistMaxSteps = 65535;     // per launch: the raw samples' tags have 17 bits
 constexpr int kPersistTablePause = 2;       // x 128 clocks between a step's preparation and its first look at the table
 constexpr int kPersistCellsPause = 4;       // x 128 clocks between clearing the tile and the first look at the cells
@@ -69,7 +75,6 @@ struct alignas(16) PersistLds {
 
 struct PersistBufs {
   unsigned long long* table;   // view [S][2 A]
-  unsigned long long* mark;    // [owners]
   unsigned long long* cells;   // 2 x [workgroups][owners][main half], then 2 x [owners][workgroups][extension]
   unsigned long long* raw;     // [N]
   unsigned* err;               // give-up word
@@ -117,7 +122,8 @@ __device__ __forceinline__ Row<8> row_of_tagged<8>(const unsigned long long (&v)
 
 // MAP = 1: the shared map staged in LDS; MAP = 2: maps read from global memory
 // (they do not change during a launch, so plain loads are fine).
-// G.n_blocks is the number of workgroups (blocks without envs hand over empty cells).
+// G.own_shift = kPersistOwnShift, G.n_blocks = 256 = the number of workgroups (blocks
+// without envs hand over empty cells).
 // Everything in B holds tag 0 at launch (cleared by the host), *B.err is zero.
 template <int A, int MAP, bool CLK>
 __global__ __launch_bounds__(256) void k_shared_persist(const Rules R, const Ptrs P, const uint64_t t0,
@@ -135,8 +141,7 @@ __global__ __launch_bounds__(256) void k_shared_persist(const Rules R, const Ptr
   const int wg = blockIdx.x;
   const int env = wg * 256 + tid;
   const bool has_env = env < P.N;
-  const int n_own = 1 << G.own_shift;  // workgroups [0, n_own) are owners, too
-  const bool is_owner = wg < n_own;
+  const int n_own = 1 << G.own_shift;  // = workgroups: every one of them is a block and an owner
 
   // a launch of this engine gave up earlier and nobody has set state and table again:
   // nothing to do (the word is read once, so that all threads take the same way)
@@ -166,14 +171,13 @@ __global__ __launch_bounds__(256) void k_shared_persist(const Rules R, const Ptr
   const DevWindow w_table = dev_window(B.table), w_cells = dev_window(B.cells);
   // 64-bit words of one buffer of main halves; cells with an extension: as many again, behind both buffers
   const size_t cells_half = ((size_t)n_own * G.n_blocks) << G.main_shift;
-  const bool has_ext = G.main_shift < G.cell_shift;
   const bool cells_flag = (R.reward_flags & 1) != 0;
   const bool base_cells = cells_flag && (R.reward_flags & 2) != 0;
 
   // owner: lane l of wave 0 keeps the table value of its key in a register; the A lanes
   // of a row sit side by side, the first of them also publishes the row's maximum
   const int own_key = key_of(wg, lane, G);
-  const bool own_live = is_owner && wave == 0 && own_key < G.K;
+  const bool own_live = wave == 0 && own_key < G.K;
   float q_own = own_live ? P.Q[own_key] : 0.0f;
   // where the lane of action a publishes: its value in the view of its cell, and the row's
   // maximum in the view of the cell that reaches this one by action a (and in its own
@@ -201,9 +205,8 @@ __global__ __launch_bounds__(256) void k_shared_persist(const Rules R, const Ptr
       if (pub_from >= 0) st_dev64(B.table + pub_from, mx);
       if (pub_self >= 0) st_dev64(B.table + pub_self, mx);
     }
-    if (lane == 0) st_dev64(B.mark + wg, tagged(0u, tag));
   };
-  if (is_owner && wave == 0) publish(1u);
+  if (wave == 0) publish(1u);
   __syncthreads();
 
   // What a step needs that does not depend on the table: computed for step k + 1 while
@@ -261,7 +264,7 @@ __global__ __launch_bounds__(256) void k_shared_persist(const Rules R, const Ptr
     CRL_MARK(0);
 
 
-    // ---- the table of this step: the view of the env's cell, one owner's mark ----------
+    // ---- the table of this step: the view of the env's cell ----------------------------
     unsigned long long rq[A], rn[A];
     {
       const uint32_t view = (uint32_t)s0 * (uint32_t)(2 * A * 8);  // byte offset of the cell's view
@@ -269,8 +272,6 @@ __global__ __launch_bounds__(256) void k_shared_persist(const Rules R, const Ptr
       int spins = 0;
       while (!ok) {
         poll_fence();
-        unsigned long long mk = tagged(0u, want);
-        if (!is_owner && tid < n_own) mk = ld_dev64(B.mark + tid);
         if (live) {
           // two units to a 16-byte load: the row, then the neighbours' maxima
 #pragma unroll
@@ -286,7 +287,7 @@ __global__ __launch_bounds__(256) void k_shared_persist(const Rules R, const Ptr
             rn[i + 1] = tagged(r.z, r.w);
           }
         }
-        ok = tag_of(mk) == want;
+        ok = true;
         if (live) {
 #pragma unroll
           for (int i = 0; i < A; ++i) ok = ok && tag_of(rq[i]) == want && tag_of(rn[i]) == want;
@@ -369,7 +370,7 @@ __global__ __launch_bounds__(256) void k_shared_persist(const Rules R, const Ptr
     CRL_MARK(3);
 
     // ---- while the cells travel: the owner's tile cleared, the next step prepared ----
-    if (is_owner) {
+    {
       float4* tile4 = reinterpret_cast<float4*>(L.tile);
 #pragma unroll
       for (int i = 0; i < kTileBlocks * kOwnKeys / 4 / 256; ++i) tile4[i * 256 + tid] = make_float4(0.0f, 0.0f, 0.0f, 0.0f);
@@ -381,93 +382,68 @@ __global__ __launch_bounds__(256) void k_shared_persist(const Rules R, const Ptr
     CRL_MARK(4);
 
     // ---- as owner of 64 keys: all blocks' cells, added in tree order --------------------
-    if (is_owner) {
-      // A wave takes 64 blocks' cells, 16 bytes = two records to a lane and load: the
-      // lanes that share a cell's main half (2 for halves of four records, up to 32) read
-      // it side by side, so a load of the wave is whole cells instead of 64 pieces of 64
-      // different ones, and the same lanes read the cell's extension.  GS loads of either
-      // at a time are asked for, checked and put into the tile: everything at once for
-      // cells of up to 16 records, eight at a time of larger ones.
+    {
+      // A wave takes 64 blocks' cells.  A main half is two pieces of 16 bytes = two records
+      // each: two lanes read it side by side, so a load of the wave is 32 whole halves, and
+      // the same two lanes read the cell's extension; all four loads are asked for at once.
       {
-        const int pc_shift = G.main_shift - 1;            // log2(pieces of a main half)
-        const int pair = lane & ((1 << pc_shift) - 1);    // this lane's piece of its cell
-        const int cells_per_load = 64 >> pc_shift;
-        const int n_loads = 1 << pc_shift;
-        const int cap_main = 1 << G.main_shift;
-        auto fetch_cells = [&](auto group_size, auto with_ext) {
-          constexpr int GS = decltype(group_size)::value;
-          constexpr bool EXT = decltype(with_ext)::value;
-          int spins = 0;
-          bool stop = false;
-          for (int j0 = 0; j0 < n_loads && !stop; j0 += GS) {
-            uint4 rec[GS], more[EXT ? GS : 1];
-            int cnt[GS];
-            uint32_t src[GS], src_more[EXT ? GS : 1];  // byte offsets into the cells
-            bool have[GS];
+        const int pair = lane & 1;  // this lane's piece of its cells
+        constexpr int GS = 2;       // loads of either kind per lane
+        int spins = 0;
+        bool stop = false;
+        uint4 rec[GS], more[GS];
+        int cnt[GS];
+        uint32_t src[GS], src_more[GS];  // byte offsets into the cells
 #pragma unroll
-            for (int j = 0; j < GS; ++j) {
-              const int blk = wave * 64 + (j0 + j) * cells_per_load + (lane >> pc_shift);
-              have[j] = blk < G.n_blocks;
-              src[j] = (uint32_t)(((size_t)half * cells_half + ((size_t)((have[j] ? blk : 0) * n_own + wg) << G.main_shift) + 2 * pair) * 8);
-              if (EXT)
-                src_more[j] = (uint32_t)(((size_t)(2 + half) * cells_half + ((size_t)(wg * G.n_blocks + (have[j] ? blk : 0)) << G.main_shift) + 2 * pair) * 8);
+        for (int j = 0; j < GS; ++j) {
+          const int blk = wave * 64 + j * 32 + (lane >> 1);
+          src[j] = (uint32_t)(((size_t)half * cells_half + ((size_t)(blk * n_own + wg) << kMainShift) + 2 * pair) * 8);
+          src_more[j] = (uint32_t)(((size_t)(2 + half) * cells_half + ((size_t)(wg * n_own + blk) << kMainShift) + 2 * pair) * 8);
+        }
+        for (;;) {
+          poll_fence();
+#pragma unroll
+          for (int j = 0; j < GS; ++j) rec[j] = ld_dev128(w_cells, src[j]);
+#pragma unroll
+          for (int j = 0; j < GS; ++j) more[j] = ld_dev128(w_cells, src_more[j]);
+          bool ok = true;
+#pragma unroll
+          for (int j = 0; j < GS; ++j) {
+            const uint32_t meta0 = (uint32_t)__shfl((int)rec[j].x, lane - pair);
+            cnt[j] = rec_count(meta0);
+            // (every record of a main half is written every step)
+            bool mine = rec_tag(meta0) == want && rec_tag(rec[j].x) == want && rec_tag(rec[j].z) == want;
+            if (cnt[j] != kSlotOverflow) {  // (an extension record: only where the count says so)
+              mine = mine && (kMainRecs + 2 * pair >= cnt[j] || rec_tag(more[j].x) == want) &&
+                     (kMainRecs + 2 * pair + 1 >= cnt[j] || rec_tag(more[j].z) == want);
             }
-            for (;;) {
-              poll_fence();
+            ok = ok && mine;
+          }
+          if (__all(ok)) break;
+          if (++spins >= spin_limit || ((spins & 63) == 0 && ld_dev32(B.err) != 0u)) {
+            L.dead = 1;
+            stop = true;
+            break;
+          }
+        }
+        if (CLK) phase_[9] += (unsigned long long)spins + 1ull;
+        __syncthreads();  // the tile is clear for everybody
+        stop = stop || L.dead != 0;
+        if (!stop) {
 #pragma unroll
-              for (int j = 0; j < GS; ++j) rec[j] = ld_dev128(w_cells, src[j]);
-              if (EXT) {
-#pragma unroll
-                for (int j = 0; j < GS; ++j) more[j] = ld_dev128(w_cells, src_more[j]);
-              }
-              bool ok = true;
-#pragma unroll
-              for (int j = 0; j < GS; ++j) {
-                const uint32_t meta0 = (uint32_t)__shfl((int)rec[j].x, lane - pair);
-                cnt[j] = rec_count(meta0);
-                // (every record of a main half is written every step)
-                bool mine = rec_tag(meta0) == want && rec_tag(rec[j].x) == want && rec_tag(rec[j].z) == want;
-                if (EXT && cnt[j] != kSlotOverflow) {  // (an extension record: only where the count says so)
-                  mine = mine && (cap_main + 2 * pair >= cnt[j] || rec_tag(more[j].x) == want) &&
-                         (cap_main + 2 * pair + 1 >= cnt[j] || rec_tag(more[j].z) == want);
-                }
-                ok = ok && (mine || !have[j]);
-              }
-              if (__all(ok)) break;
-              if (++spins >= spin_limit || ((spins & 63) == 0 && ld_dev32(B.err) != 0u)) {
-                L.dead = 1;
-                stop = true;
-                break;
-              }
-            }
-            if (j0 == 0) {
-              if (CLK) phase_[9] += (unsigned long long)spins + 1ull;
-              __syncthreads();  // the tile is clear for everybody
-              stop = stop || L.dead != 0;
-            }
-            if (stop) break;
-#pragma unroll
-            for (int j = 0; j < GS; ++j) {
-              const int blk = wave * 64 + (j0 + j) * cells_per_load + (lane >> pc_shift);
-              if (have[j]) {
-                float* row = L.tile + blk * kOwnKeys;
-                if (cnt[j] == kSlotOverflow) {
-                  if (pair == 0) L.o_list[atomicAdd(&L.o_count, 1)] = (uint8_t)blk;
-                } else {
-                  if (2 * pair < cnt[j]) row[rec_slot(rec[j].x)] = __uint_as_float(rec[j].y);
-                  if (2 * pair + 1 < cnt[j]) row[rec_slot(rec[j].z)] = __uint_as_float(rec[j].w);
-                  if (EXT) {
-                    if (cap_main + 2 * pair < cnt[j]) row[rec_slot(more[j].x)] = __uint_as_float(more[j].y);
-                    if (cap_main + 2 * pair + 1 < cnt[j]) row[rec_slot(more[j].z)] = __uint_as_float(more[j].w);
-                  }
-                }
-              }
+          for (int j = 0; j < GS; ++j) {
+            const int blk = wave * 64 + j * 32 + (lane >> 1);
+            float* row = L.tile + blk * kOwnKeys;
+            if (cnt[j] == kSlotOverflow) {
+              if (pair == 0) L.o_list[atomicAdd(&L.o_count, 1)] = (uint8_t)blk;
+            } else {
+              if (2 * pair < cnt[j]) row[rec_slot(rec[j].x)] = __uint_as_float(rec[j].y);
+              if (2 * pair + 1 < cnt[j]) row[rec_slot(rec[j].z)] = __uint_as_float(rec[j].w);
+              if (kMainRecs + 2 * pair < cnt[j]) row[rec_slot(more[j].x)] = __uint_as_float(more[j].y);
+              if (kMainRecs + 2 * pair + 1 < cnt[j]) row[rec_slot(more[j].z)] = __uint_as_float(more[j].w);
             }
           }
-        };
-        if (has_ext && n_loads == 2) fetch_cells(std::integral_constant<int, 2>{}, std::true_type{});
-        else if (has_ext && n_loads == 4) fetch_cells(std::integral_constant<int, 4>{}, std::true_type{});
-        else fetch_cells(std::integral_constant<int, 8>{}, std::false_type{});
+        }
       }
       CRL_MARK(5);
       __syncthreads();

@@ -382,17 +382,16 @@ def test_shared_table_one_launch_kernel_shapes(gpu, oracle):
     of envs (workgroups without envs), a last block that is not full, 8 actions
     with per-cell rewards and per-env maps read from global memory, calls that
     alternate (chunked launches)."""
-    # 300 envs = 2 blocks, 1024 keys = 16 owners
+    # 300 envs = 2 of 256 blocks with envs, 1024 keys = 4 to an owner
     cls, start = gpu.gen_maps_bernoulli(5, 1, 300, 16, 16, 0.1, 0.03)
     cfg = gpu.make_config(300, 16, 16, table_mode=gpu.TABLE_SHARED, map_mode=gpu.MAP_SHARED, lr=0.01, eps0=0.3,
                           episode_len=25, seed=3, trap_reward=-0.5)
     with gpu.Engine(cfg, 0) as eng:
-        # automatic: two launches per step for a table this small (16 owners)
-        assert eng.fused_kernel_info(10)["name"] == "k_shared_act+k_reduce_owners"
+        assert eng.fused_kernel_info(10)["name"] == "k_shared_persist<4,1>"  # (automatic)
         eng.set_fused_variant(1)
         assert eng.fused_kernel_info(10)["name"] == "k_shared_act+k_reduce_owners"
         eng.set_fused_variant(2)
-        assert eng.fused_kernel_info(1)["name"] == "k_shared_persist<4,1>" and eng.fused_kernel_info(1)["grid"] == 16
+        assert eng.fused_kernel_info(1)["name"] == "k_shared_persist<4,1>" and eng.fused_kernel_info(1)["grid"] == 256
     run_both(gpu, oracle, cfg, cls, start, 90, chunks=[1, 30, 1, 1, 50, 7], variant=2)
     # 8 actions, cell rewards, per-env maps (global memory), linear epsilon, 1000 envs: last block 232 envs
     N, W, H = 1000, 24, 20
@@ -484,11 +483,12 @@ def test_shared_table_one_launch_kernel_gives_up_cleanly(gpu):
 
 
 def test_shared_table_automatic_plan_and_cell_sizes(gpu, oracle):
-    """What crl_run_fused picks by itself, and the hand-off cells of every size: 8
-    records (256 owners), 16 (64 owners), 32 (32 owners), 64 (16 owners and fewer), each
-    through the one-launch kernel and through two launches per step."""
-    for N, W, H, auto in ((3000, 64, 64, "persist"), (3000, 32, 32, "persist"), (3000, 32, 16, "two"), (3000, 16, 16, "two"),
-                          (700, 5, 5, "two")):
+    """What crl_run_fused picks by itself, and tables of every size: through the one-launch
+    kernel (always 256 owners: 64 keys each down to none) and through two launches per
+    step (hand-off cells of 8 records for 256 owners, 16 for 64, 32 for 32, 64 for 16 and
+    fewer)."""
+    for N, W, H, auto in ((3000, 64, 64, "persist"), (3000, 32, 32, "persist"), (3000, 32, 16, "persist"),
+                          (3000, 16, 16, "persist"), (700, 5, 5, "persist")):
         cls, start = gpu.gen_maps_bernoulli(9, 1, N, W, H, 0.12, 0.03)
         cfg = gpu.make_config(N, W, H, table_mode=gpu.TABLE_SHARED, map_mode=gpu.MAP_SHARED, lr=0.003, eps0=0.3,
                               episode_len=30, seed=4, trap_reward=-0.5)
