@@ -134,11 +134,11 @@ int crl_set_resident_envs(crl_engine* e, int32_t n_envs);
  * Per-env tables: 1 = plain (every wave steps envs against tables in HBM),
  * 2 = hybrid (the last wave of each workgroup steps envs whose whole tables it holds
  * in LDS; used only when 32 tables fit; automatic picks it for launches of at
- * least 64 steps).  Shared table: 0 and 1 = two launches per step, 2 = all steps of
- * a call in one launch whose workgroups exchange block sums and table values through
- * device-scope loads and stores (needs every workgroup resident at once: at most
- * 65,536 envs and 16,384 table entries, else two launches per step; slower than
- * those on MI355X, kept for callers that must not launch per step).
+ * least 64 steps).  Shared table: 1 = two launches per step; 2 = all steps of a
+ * call in one launch whose 256 workgroups exchange block sums and table values
+ * through device-scope loads and stores (needs every workgroup resident at once:
+ * at most 65,536 envs and 16,384 table entries, else two launches per step);
+ * automatic picks the one launch for calls of at least 4 steps.
  * Results do not depend on it. */
 int crl_set_fused_variant(crl_engine* e, int32_t variant);
 /* How the last hybrid crl_run_fused split the envs between its two kinds of
@@ -211,7 +211,7 @@ int crl_run_fused(crl_engine* e, int32_t n_steps);
  * until the process ends, and the call allocates and frees nothing (device or
  * host).  CRL_E_RANGE if the engine's ordered reduction needs more hand-off cells
  * than the array holds (65,536 envs on a 64x64x4 table need 4 MB with two launches
- * per step, 9.2 MB of exchange buffers in the one-launch kernel; an engine whose
+ * per step, 9.7 MB of exchange buffers in the one-launch kernel; an engine whose
  * one-launch buffers do not fit takes two launches per step).  All engines on one GPU share that GPU's
  * array: calls that overlap in time on one GPU (different streams or threads)
  * race; calls in stream order do not. */
