@@ -194,3 +194,38 @@ def test_random_configs_general(gpu, oracle, seed):
         assert same(q, st, Q, ost), what
         if trace_n:
             assert all(np.array_equal(tr[k], want[k]) for k in ("s_next", "action", "reward", "done")), what
+
+
+@pytest.mark.parametrize("seed", [7, 8])
+def test_random_configs_shared_table(gpu, oracle, seed):
+    """One shared table under the ordered reduction at every size of table and batch the
+    one-launch kernel takes (3x3 to 64x64 cells, 300 to 65,536 envs, learning rates from
+    tame to diverging, episodes of one step to none), through one launch per call and
+    through two launches per step, calls split at a random step."""
+    rng = np.random.default_rng(seed)
+    for case in range(12):
+        A = int(rng.choice([4, 4, 8]))
+        W, H = int(rng.integers(3, 65)), int(rng.integers(3, 65))
+        while W * H * A > 16384:
+            H = max(3, H // 2)
+        N = int(rng.choice([300, 1000, 5000, 20000, 65536]))
+        lr = float(rng.choice([0.0005, 0.01, 0.05, 0.3]))
+        steps = int(rng.integers(20, 120)) if N > 20000 else int(rng.integers(50, 300))
+        cls, start = gpu.gen_maps_bernoulli(int(rng.integers(1, 99)), 1, N, W, H, float(rng.uniform(0, 0.25)),
+                                            float(rng.uniform(0, 0.05)))
+        cfg = gpu.make_config(N, W, H, n_actions=A, table_mode=gpu.TABLE_SHARED, map_mode=gpu.MAP_SHARED, lr=lr,
+                              eps0=float(rng.uniform(0.05, 1.0)), episode_len=int(rng.choice([0, 1, 7, 40])),
+                              seed=int(rng.integers(1, 1000)), trap_reward=-0.5)
+        first = int(rng.integers(1, steps))
+        variant = 1 if case % 4 == 3 else 2
+        with gpu.Engine(cfg, 0) as eng:
+            eng.set_maps(cls, start)
+            eng.set_fused_variant(variant)
+            name = eng.fused_kernel_info(first)["name"]
+            eng.run_fused(first)
+            eng.run_fused(steps - first)
+            q, st = eng.q_get(0, 1), eng.get_state()
+        Q = np.zeros((1, W * H, A), np.float32)
+        ost = oracle.new_state(cfg, start)
+        oracle.run(cfg, cls, None, start, Q, ost, 0, steps)
+        assert same(q, st, Q, ost), (seed, case, name, A, W, H, N, lr, steps, first)
