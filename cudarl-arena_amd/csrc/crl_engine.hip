@@ -135,8 +135,8 @@ struct crl_engine {
   unsigned* tk = nullptr;  // ticket counters {next ticket, envs on HBM tables, envs on LDS tables}
   bool split_valid = false;  // the last fused launch drew tickets
   unsigned long long* ho = nullptr;  // hand-off cells of the ordered reduction
-  // one-launch shared-table kernel: what its workgroups exchange (tagged table, row
-  // maxima, marks, raw samples, hand-off cells), the engine's own give-up word
+  // one-launch shared-table kernel: what its workgroups exchange (the tagged views of
+  // the table's cells, raw samples, hand-off cells), the engine's own give-up word
   // followed by the phase clocks, and whether a launch has not been checked for
   // having given up yet
   DevBuf<unsigned long long> pbuf;

@@ -9,9 +9,10 @@
 // Two passes over the chip:
 //   1. one workgroup per block: the lowest thread that holds a key becomes the
 //      key's leader (LDS atomic min on a dense table), the other holders mark
-//      themselves in the leader's 256-bit member set (LDS atomic or), and the
-//      leader adds the members' deltas in thread order = sample order; every
-//      distinct key's block sum goes to the workgroup that owns the key;
+//      themselves in the leader's 256-bit member set (LDS atomic or) and line
+//      their deltas up by their place in it, and the leader adds them in that
+//      order = thread order = sample order; every distinct key's block sum goes
+//      to the workgroup that owns the key;
 //   2. one workgroup per 64 keys lays the block sums it was handed out as a
 //      dense [block][key] tile in LDS and adds the columns in the tree order.
 // Empty blocks add +0.0f, which changes nothing, so the result is a pure
@@ -27,7 +28,7 @@ constexpr int kGroupBlocks = 16;     // level 1
 constexpr int kOwnKeys = 64;         // keys per owner workgroup: 64 / A whole table rows
 constexpr int kMinCellRecs = 8;      // records of a hand-off cell: 8 ... 64, see cell_shift_for()
 constexpr int kSlotOverflow = 127;   // count value: more distinct keys than records, read the block's raw samples instead
-constexpr int kStagePieces = 1024;   // 16-byte pieces of one block's cells at most: owners x records / 2
+constexpr int kStagePieces = 1024;   // 16-byte pieces of the main halves of one block's cells at most
 constexpr int kDenseKeys = 16384;    // keys the dense LDS table of pass 1 can hold
 constexpr int kTileBlocks = 256;     // blocks per LDS tile of pass 2
 constexpr uint32_t kOwnerMix = 37;   // odd: spreads cells a power of two apart over owners
