@@ -64,7 +64,9 @@ constexpr int kPersistClockWords = 20 + 8 * 256;  // 2 workgroups x (8 phases + 
 
 struct alignas(16) PersistLds {
   ReduceLds red;
-  alignas(16) float tile[kTileBlocks * kOwnKeys];       // the owner's [block][key] block sums (cleared 16 bytes at a time)
+  alignas(16) float tile[kTileBlocks * kOwnKeys];       // the owner's [block][key] block sums: a quarter (64 blocks) to a wave, which
+                                                        // clears, fills and adds up its quarter without waiting for the others
+  alignas(16) unsigned long long stage[kPersistMaxGroups << kMainShift];  // the main halves of the block's cells on their way out
   float gsum[(kTileBlocks / kGroupBlocks) * kOwnKeys];  // [group][key]
   float o_delta[kBlockSamples];                         // raw samples of one overflowing block
   uint8_t o_slot[kBlockSamples];
@@ -133,7 +135,7 @@ __global__ __launch_bounds__(256) void k_shared_persist(const Rules R, const Ptr
   extern __shared__ __align__(16) unsigned char lds_raw[];
   PersistLds& L = *reinterpret_cast<PersistLds*>(lds_raw);
   static_assert(sizeof(PersistLds) % 16 == 0 && offsetof(PersistLds, tile) % 16 == 0, "16-byte LDS accesses");
-  static_assert(kStagePieces * 16 + kSortBytes <= sizeof(L.tile), "cell staging and the holders' line-up share the tile");
+  static_assert(kSortBytes <= sizeof(L.tile) / 2, "the holders' line-up borrows the upper half of the tile");
   uint32_t* lds_map = reinterpret_cast<uint32_t*>(lds_raw + sizeof(PersistLds));
   const int tid = threadIdx.x;
   const int lane = tid & 63;
@@ -255,7 +257,7 @@ __global__ __launch_bounds__(256) void k_shared_persist(const Rules R, const Ptr
     CRL_MARK(7);
     // (the values this workgroup published as an owner are on their way meanwhile)
     prepare(k);
-    reduce_stage_init(reinterpret_cast<unsigned long long*>(L.tile), G, want);
+    reduce_stage_init(L.stage, G, want);
     // A first look that comes too early costs a whole round trip more than one that comes
     // just in time: the values published at the end of the last step need about 1.5 us to
     // be visible, the preparation above takes 1 us (65,536 envs on 64x64x4, us per step by
@@ -360,9 +362,9 @@ __global__ __launch_bounds__(256) void k_shared_persist(const Rules R, const Ptr
 
     // ---- block sums to the owners' cells ------------------------------------------------
     const int half = k & 1;  // cells and raw samples: two buffers, taken in turn
-    // (`sorted`: the upper half of the tile; the staging area of the cells is in its first 8 KB)
+    // (`sorted`: the upper half of the tile, which is free until the block sums are through)
     const bool over = reduce_block<true>(L.red, G, wg, my_key, my_delta, live, B.cells, want, L.tile + kTileBlocks * kOwnKeys / 2,
-                                         reinterpret_cast<unsigned long long*>(L.tile), &w_cells,
+                                         L.stage, &w_cells,
                                          (uint32_t)((size_t)half * cells_half * 8), B.cells + (2 + half) * cells_half);
     if (over && has_env)
       st_dev64(B.raw + (size_t)half * P.N + env, tagged(__float_as_uint(my_delta),
@@ -370,10 +372,10 @@ __global__ __launch_bounds__(256) void k_shared_persist(const Rules R, const Ptr
     CRL_MARK(3);
 
     // ---- while the cells travel: the owner's tile cleared, the next step prepared ----
-    {
-      float4* tile4 = reinterpret_cast<float4*>(L.tile);
+    {  // (each wave its own quarter)
+      float4* tile4 = reinterpret_cast<float4*>(L.tile) + wave * (kTileBlocks * kOwnKeys / 4 / 4);
 #pragma unroll
-      for (int i = 0; i < kTileBlocks * kOwnKeys / 4 / 256; ++i) tile4[i * 256 + tid] = make_float4(0.0f, 0.0f, 0.0f, 0.0f);
+      for (int i = 0; i < kTileBlocks * kOwnKeys / 4 / 256; ++i) tile4[i * 64 + lane] = make_float4(0.0f, 0.0f, 0.0f, 0.0f);
     }
     // A short pause before the first look at the others' cells: asking while the own
     // stores have only just left takes longer (no pause 7.06 us per step, 4 x 128 clocks
@@ -427,8 +429,6 @@ __global__ __launch_bounds__(256) void k_shared_persist(const Rules R, const Ptr
           }
         }
         if (CLK) phase_[9] += (unsigned long long)spins + 1ull;
-        __syncthreads();  // the tile is clear for everybody
-        stop = stop || L.dead != 0;
         if (!stop) {
 #pragma unroll
           for (int j = 0; j < GS; ++j) {
@@ -446,50 +446,66 @@ __global__ __launch_bounds__(256) void k_shared_persist(const Rules R, const Ptr
         }
       }
       CRL_MARK(5);
+      // the wave's four groups: its own 64 rows of the tile, which only it has written
+      auto group_sums = [&]() {
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+        __builtin_amdgcn_wave_barrier();
+        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+#pragma unroll
+        for (int gi = 0; gi < 4; ++gi) {
+          const int grp = wave * 4 + gi;
+          float acc = 0.0f;
+#pragma unroll
+          for (int bb = 0; bb < kGroupBlocks; ++bb) acc = acc + L.tile[(grp * kGroupBlocks + bb) * kOwnKeys + lane];
+          L.gsum[grp * kOwnKeys + lane] = acc;
+        }
+      };
+      group_sums();
       __syncthreads();
       if (L.dead) {  // some wave gave up waiting for its cells
         gave_up = true;
         break;
       }
-      // blocks with more distinct keys for this owner than a cell holds: their raw
-      // samples, all threads at once, then one thread per key adds its matches in order
+      // blocks with more distinct keys for this owner than a cell holds (rare): their raw
+      // samples, all threads at once, then one thread per key adds its matches in order,
+      // and the group sums once more
       const int n_over = L.o_count;
-      bool raw_failed = false;
-      for (int q = 0; q < n_over; ++q) {
-        const int bb = L.o_list[q];
-        const int i = bb * kBlockSamples + tid;
-        int slot = 255;
-        float dv = 0.0f;
-        if (i < P.N) {
-          unsigned long long v = 0ull;
-          int spins = 0;
-          for (;;) {
-            poll_fence();
-            v = ld_dev64(B.raw + (size_t)half * P.N + i);
-            if ((tag_of(v) >> kRawTagShift) == want) break;
-            if (++spins >= spin_limit || ((spins & 63) == 0 && ld_dev32(B.err) != 0u)) {
-              raw_failed = true;
-              break;
+      if (n_over > 0) {
+        bool raw_failed = false;
+        for (int q = 0; q < n_over; ++q) {
+          const int bb = L.o_list[q];
+          const int i = bb * kBlockSamples + tid;
+          int slot = 255;
+          float dv = 0.0f;
+          if (i < P.N) {
+            unsigned long long v = 0ull;
+            int spins = 0;
+            for (;;) {
+              poll_fence();
+              v = ld_dev64(B.raw + (size_t)half * P.N + i);
+              if ((tag_of(v) >> kRawTagShift) == want) break;
+              if (++spins >= spin_limit || ((spins & 63) == 0 && ld_dev32(B.err) != 0u)) {
+                raw_failed = true;
+                break;
+              }
+            }
+            const int kk = (int)(tag_of(v) & kRawKeyMask);
+            if (!raw_failed && (tag_of(v) & kRawValid) && owner_of(kk, G) == wg) {
+              slot = slot_of(kk, G);
+              dv = value_of(v);
             }
           }
-          const int kk = (int)(tag_of(v) & kRawKeyMask);
-          if (!raw_failed && (tag_of(v) & kRawValid) && owner_of(kk, G) == wg) {
-            slot = slot_of(kk, G);
-            dv = value_of(v);
+          L.o_slot[tid] = (uint8_t)slot;
+          L.o_delta[tid] = dv;
+          __syncthreads();
+          if (tid < kOwnKeys) {
+            float acc = 0.0f;
+            for (int j = 0; j < kBlockSamples; ++j)
+              if (L.o_slot[j] == tid) acc = acc + L.o_delta[j];  // sample order
+            L.tile[bb * kOwnKeys + tid] = acc;
           }
+          __syncthreads();
         }
-        L.o_slot[tid] = (uint8_t)slot;
-        L.o_delta[tid] = dv;
-        __syncthreads();
-        if (tid < kOwnKeys) {
-          float acc = 0.0f;
-          for (int j = 0; j < kBlockSamples; ++j)
-            if (L.o_slot[j] == tid) acc = acc + L.o_delta[j];  // sample order
-          L.tile[bb * kOwnKeys + tid] = acc;
-        }
-        __syncthreads();
-      }
-      if (n_over > 0) {
         if (tid == 0) L.o_count = 0;
         if (raw_failed) L.dead = 1;
         __syncthreads();
@@ -497,16 +513,9 @@ __global__ __launch_bounds__(256) void k_shared_persist(const Rules R, const Ptr
           gave_up = true;
           break;
         }
+        group_sums();
+        __syncthreads();
       }
-#pragma unroll
-      for (int gi = 0; gi < 4; ++gi) {
-        const int grp = wave * 4 + gi;
-        float acc = 0.0f;
-#pragma unroll
-        for (int bb = 0; bb < kGroupBlocks; ++bb) acc = acc + L.tile[(grp * kGroupBlocks + bb) * kOwnKeys + lane];
-        L.gsum[grp * kOwnKeys + lane] = acc;
-      }
-      __syncthreads();
       if (wave == 0) {
         float total = 0.0f;
 #pragma unroll
