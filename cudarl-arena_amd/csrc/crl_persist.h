@@ -300,11 +300,9 @@ __global__ __launch_bounds__(256) void k_shared_persist(const Rules R, const Ptr
         }
       }
       if (CLK) phase_[8] += (unsigned long long)spins + 1ull;
-      __syncthreads();
-      if (L.dead) {
-        gave_up = true;
-        break;
-      }
+      // (no barrier here: the block sums begin with one, behind which every thread of the
+      // workgroup has read its view - cells are written later still - and whether some
+      // thread gave up is looked at behind them; until then it works on whatever it got)
     }
     CRL_MARK(1);
 
@@ -366,6 +364,10 @@ __global__ __launch_bounds__(256) void k_shared_persist(const Rules R, const Ptr
     const bool over = reduce_block<true>(L.red, G, wg, my_key, my_delta, live, B.cells, want, L.tile + kTileBlocks * kOwnKeys / 2,
                                          L.stage, &w_cells,
                                          (uint32_t)((size_t)half * cells_half * 8), B.cells + (2 + half) * cells_half);
+    if (L.dead) {  // some thread gave up waiting for the table
+      gave_up = true;
+      break;
+    }
     if (over && has_env)
       st_dev64(B.raw + (size_t)half * P.N + env, tagged(__float_as_uint(my_delta),
                                    (uint32_t)my_key | (live ? kRawValid : 0u) | (want << kRawTagShift)));
