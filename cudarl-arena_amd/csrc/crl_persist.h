@@ -195,11 +195,18 @@ __global__ __launch_bounds__(256) void k_shared_persist(const Rules R, const Ptr
     if (!((unsigned)(x + dx) < (unsigned)R.W && (unsigned)(y + dy) < (unsigned)R.H)) pub_self = c * 2 * A + A + a;
   }
   auto publish = [&](uint32_t tag) {  // wave 0 of an owner
+    if (own_live) st_dev64(B.table + pub_q, tagged(__float_as_uint(q_own), tag));
     float qs[A];
+    if constexpr (A == 4) {  // the four lanes of a row are a quad: a move within it, no trip through LDS
+      qs[0] = __int_as_float(__builtin_amdgcn_mov_dpp(__float_as_int(q_own), 0x00, 0xf, 0xf, true));
+      qs[1] = __int_as_float(__builtin_amdgcn_mov_dpp(__float_as_int(q_own), 0x55, 0xf, 0xf, true));
+      qs[2] = __int_as_float(__builtin_amdgcn_mov_dpp(__float_as_int(q_own), 0xaa, 0xf, 0xf, true));
+      qs[3] = __int_as_float(__builtin_amdgcn_mov_dpp(__float_as_int(q_own), 0xff, 0xf, 0xf, true));
+    } else {
 #pragma unroll
-    for (int i = 0; i < A; ++i) qs[i] = __shfl(q_own, (lane & ~(A - 1)) + i);
+      for (int i = 0; i < A; ++i) qs[i] = __shfl(q_own, (lane & ~(A - 1)) + i);
+    }
     if (own_live) {
-      st_dev64(B.table + pub_q, tagged(__float_as_uint(q_own), tag));
       Row<A> row;
       if constexpr (A == 4) row = Row<4>{qs[0], qs[1], qs[2], qs[3]};
       else row = Row<8>{qs[0], qs[1], qs[2], qs[3], qs[4], qs[5], qs[6], qs[7]};
@@ -364,10 +371,6 @@ __global__ __launch_bounds__(256) void k_shared_persist(const Rules R, const Ptr
     const bool over = reduce_block<true>(L.red, G, wg, my_key, my_delta, live, B.cells, want, L.tile + kTileBlocks * kOwnKeys / 2,
                                          L.stage, &w_cells,
                                          (uint32_t)((size_t)half * cells_half * 8), B.cells + (2 + half) * cells_half);
-    if (L.dead) {  // some thread gave up waiting for the table
-      gave_up = true;
-      break;
-    }
     if (over && has_env)
       st_dev64(B.raw + (size_t)half * P.N + env, tagged(__float_as_uint(my_delta),
                                    (uint32_t)my_key | (live ? kRawValid : 0u) | (want << kRawTagShift)));
@@ -383,6 +386,10 @@ __global__ __launch_bounds__(256) void k_shared_persist(const Rules R, const Ptr
     // stores have only just left takes longer (no pause 7.06 us per step, 4 x 128 clocks
     // 6.97, 8 x 7.03, 12 x 7.56; waiting until the 8 KB of own cells are acknowledged 7.30).
     for (int i = 0; i < kPersistCellsPause; ++i) __builtin_amdgcn_s_sleep(2);
+    if (L.dead) {  // some thread gave up waiting for the table
+      gave_up = true;
+      break;
+    }
     CRL_MARK(4);
 
     // ---- as owner of 64 keys: all blocks' cells, added in tree order --------------------
@@ -464,6 +471,14 @@ __global__ __launch_bounds__(256) void k_shared_persist(const Rules R, const Ptr
       };
       group_sums();
       __syncthreads();
+      // (the totals are asked for along with the two words that say whether they stand)
+      auto totals = [&]() {
+        float total = 0.0f;
+#pragma unroll
+        for (int grp = 0; grp < kTileBlocks / kGroupBlocks; ++grp) total = total + L.gsum[grp * kOwnKeys + lane];
+        return total;
+      };
+      float total = totals();
       if (L.dead) {  // some wave gave up waiting for its cells
         gave_up = true;
         break;
@@ -517,11 +532,9 @@ __global__ __launch_bounds__(256) void k_shared_persist(const Rules R, const Ptr
         }
         group_sums();
         __syncthreads();
+        total = totals();
       }
       if (wave == 0) {
-        float total = 0.0f;
-#pragma unroll
-        for (int grp = 0; grp < kTileBlocks / kGroupBlocks; ++grp) total = total + L.gsum[grp * kOwnKeys + lane];
         q_own = q_own + total;
         publish(want + 1u);
       }
