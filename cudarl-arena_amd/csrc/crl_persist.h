@@ -420,7 +420,8 @@ __global__ __launch_bounds__(256) void k_shared_persist(const Rules R, const Ptr
           bool ok = true;
 #pragma unroll
           for (int j = 0; j < GS; ++j) {
-            const uint32_t meta0 = (uint32_t)__shfl((int)rec[j].x, lane - pair);
+            // (record 0 of the cell is in the even lane of the two: a move within the quad)
+            const uint32_t meta0 = (uint32_t)__builtin_amdgcn_mov_dpp((int)rec[j].x, 0xa0, 0xf, 0xf, true);
             cnt[j] = rec_count(meta0);
             // (every record of a main half is written every step)
             bool mine = rec_tag(meta0) == want && rec_tag(rec[j].x) == want && rec_tag(rec[j].z) == want;
