@@ -55,7 +55,8 @@ constexpr int kPersistMaxGroups = 256;      // workgroups: one per compute unit,
 constexpr int kPersistOwnShift = 8;         // log2(owners): always 256, every workgroup is one
 constexpr int kMainShift = 2, kMainRecs = 1 << kMainShift;  // records in the half of a cell that is written every step
 static_assert(main_shift_for(kPersistOwnShift) == kMainShift && cell_shift_for(kPersistOwnShift) == kMainShift + 1 &&
-              (1 << kPersistOwnShift) == kPersistMaxGroups, "the owner's loads are laid out for cells of 4 + 4 records");
+              (1 << kPersistOwnShift) == kPersistMaxGroups && (kPersistMaxGroups << (kMainShift - 1)) == kStagePieces,
+              "the owner's loads are laid out for cells of 4 + 4 records");
 constexpr int kPersistMaxSteps = 65535;     // per launch: the raw samples' tags have 17 bits
 constexpr int kPersistTablePause = 2;       // x 128 clocks between a step's preparation and its first look at the table
 constexpr int kPersistCellsPause = 4;       // x 128 clocks between clearing the tile and the first look at the cells

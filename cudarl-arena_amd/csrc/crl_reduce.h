@@ -28,7 +28,7 @@ constexpr int kGroupBlocks = 16;     // level 1
 constexpr int kOwnKeys = 64;         // keys per owner workgroup: 64 / A whole table rows
 constexpr int kMinCellRecs = 8;      // records of a hand-off cell: 8 ... 64, see cell_shift_for()
 constexpr int kSlotOverflow = 127;   // count value: more distinct keys than records, read the block's raw samples instead
-constexpr int kStagePieces = 1024;   // 16-byte pieces of the main halves of one block's cells at most
+constexpr int kStagePieces = 512;    // 16-byte pieces of the main halves of one block's cells in the one-launch kernel
 constexpr int kDenseKeys = 16384;    // keys the dense LDS table of pass 1 can hold
 constexpr int kTileBlocks = 256;     // blocks per LDS tile of pass 2
 constexpr uint32_t kOwnerMix = 37;   // odd: spreads cells a power of two apart over owners
@@ -293,11 +293,13 @@ __device__ __forceinline__ bool reduce_block(ReduceLds& L, const ReduceGeom G, c
              make_rec((uint32_t)slot_of(key, G), 0u, tag, acc));
 
   if (DEV) {
-    // (at most kStagePieces pieces = four to a thread, all asked for before the first is used)
+    // (the one-launch kernel always has 256 owners and main halves of 4 records: 512 pieces,
+    // two to a thread, both asked for before the first is used)
     const ulonglong2* stage2 = reinterpret_cast<const ulonglong2*>(stage);
     const int piece_shift = G.main_shift - 1;  // log2(pieces of a cell's main half)
     const int pieces = n_own << piece_shift;
     constexpr int kPer = kStagePieces / kBlockSamples;
+    static_assert(kPer == 2, "two pieces of the stage to a thread");
     ulonglong2 v[kPer];
     int c[kPer];
 #pragma unroll
