@@ -68,7 +68,7 @@ struct alignas(16) PersistLds {
   alignas(16) float tile[kTileBlocks * kOwnKeys];       // the owner's [block][key] block sums: a quarter (64 blocks) to a wave, which
                                                         // clears, fills and adds up its quarter without waiting for the others
   alignas(16) unsigned long long stage[kPersistMaxGroups << kMainShift];  // the main halves of the block's cells on their way out
-  float gsum[(kTileBlocks / kGroupBlocks) * kOwnKeys];  // [group][key]
+  alignas(16) float gsum[(kTileBlocks / kGroupBlocks) * kOwnKeys];  // [group][key] (written 16 bytes at a time)
   float o_delta[kBlockSamples];                         // raw samples of one overflowing block
   uint8_t o_slot[kBlockSamples];
   uint8_t o_list[kTileBlocks];  // blocks whose cell overflowed this step
@@ -462,14 +462,21 @@ __global__ __launch_bounds__(256) void k_shared_persist(const Rules R, const Ptr
         __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
         __builtin_amdgcn_wave_barrier();
         __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+        // a lane takes four keys of one of the wave's four groups: 16 loads of 16 bytes
+        const int grp = wave * 4 + (lane >> 4);
+        const float4* rows = reinterpret_cast<const float4*>(L.tile + grp * kGroupBlocks * kOwnKeys) + (lane & 15);
+        float4 v[kGroupBlocks];
 #pragma unroll
-        for (int gi = 0; gi < 4; ++gi) {
-          const int grp = wave * 4 + gi;
-          float acc = 0.0f;
+        for (int bb = 0; bb < kGroupBlocks; ++bb) v[bb] = rows[bb * (kOwnKeys / 4)];
+        float4 acc = make_float4(0.0f, 0.0f, 0.0f, 0.0f);
 #pragma unroll
-          for (int bb = 0; bb < kGroupBlocks; ++bb) acc = acc + L.tile[(grp * kGroupBlocks + bb) * kOwnKeys + lane];
-          L.gsum[grp * kOwnKeys + lane] = acc;
+        for (int bb = 0; bb < kGroupBlocks; ++bb) {
+          acc.x = acc.x + v[bb].x;
+          acc.y = acc.y + v[bb].y;
+          acc.z = acc.z + v[bb].z;
+          acc.w = acc.w + v[bb].w;
         }
+        reinterpret_cast<float4*>(L.gsum + grp * kOwnKeys)[lane & 15] = acc;
       };
       group_sums();
       __syncthreads();
