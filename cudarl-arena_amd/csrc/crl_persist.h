@@ -58,8 +58,8 @@ static_assert(main_shift_for(kPersistOwnShift) == kMainShift && cell_shift_for(k
               (1 << kPersistOwnShift) == kPersistMaxGroups && (kPersistMaxGroups << (kMainShift - 1)) == kStagePieces,
               "the owner's loads are laid out for cells of 4 + 4 records");
 constexpr int kPersistMaxSteps = 65535;     // per launch: the raw samples' tags have 17 bits
-constexpr int kPersistTablePause = 2;       // x 128 clocks between a step's preparation and its first look at the table
-constexpr int kPersistCellsPause = 4;       // x 128 clocks between clearing the tile and the first look at the cells
+constexpr int kPersistTablePause = 1;       // x 128 clocks between a step's preparation and its first look at the table
+constexpr int kPersistCellsPause = 1;       // x 128 clocks between clearing the tile and the first look at the cells
 constexpr int kPersistClockWords = 20 + 8 * 256;  // 2 workgroups x (8 phases + polls of the two waits by thread 0),
                                                   // then the wall clock of every workgroup at the 8 marks of one step
 
