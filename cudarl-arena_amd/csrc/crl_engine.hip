@@ -540,14 +540,22 @@ int opt_in_lds(crl_engine* e) {
   HIP_TRY(allow_lds(crl::k_shared_act<4, 2, true>, act - kStaticLdsReserve));
   HIP_TRY(allow_lds(crl::k_shared_act<8, 1, true>, act - kStaticLdsReserve));
   HIP_TRY(allow_lds(crl::k_shared_act<8, 2, true>, act - kStaticLdsReserve));
-  HIP_TRY(allow_lds(crl::k_shared_persist<4, 1, false>, act - kStaticLdsReserve));
-  HIP_TRY(allow_lds(crl::k_shared_persist<4, 2, false>, act - kStaticLdsReserve));
-  HIP_TRY(allow_lds(crl::k_shared_persist<8, 1, false>, act - kStaticLdsReserve));
-  HIP_TRY(allow_lds(crl::k_shared_persist<8, 2, false>, act - kStaticLdsReserve));
-  HIP_TRY(allow_lds(crl::k_shared_persist<4, 1, true>, act - kStaticLdsReserve));
-  HIP_TRY(allow_lds(crl::k_shared_persist<4, 2, true>, act - kStaticLdsReserve));
-  HIP_TRY(allow_lds(crl::k_shared_persist<8, 1, true>, act - kStaticLdsReserve));
-  HIP_TRY(allow_lds(crl::k_shared_persist<8, 2, true>, act - kStaticLdsReserve));
+  HIP_TRY(allow_lds(crl::k_shared_persist<4, 1, false, false>, act - kStaticLdsReserve));
+  HIP_TRY(allow_lds(crl::k_shared_persist<4, 1, false, true>, act - kStaticLdsReserve));
+  HIP_TRY(allow_lds(crl::k_shared_persist<4, 2, false, false>, act - kStaticLdsReserve));
+  HIP_TRY(allow_lds(crl::k_shared_persist<4, 2, false, true>, act - kStaticLdsReserve));
+  HIP_TRY(allow_lds(crl::k_shared_persist<8, 1, false, false>, act - kStaticLdsReserve));
+  HIP_TRY(allow_lds(crl::k_shared_persist<8, 1, false, true>, act - kStaticLdsReserve));
+  HIP_TRY(allow_lds(crl::k_shared_persist<8, 2, false, false>, act - kStaticLdsReserve));
+  HIP_TRY(allow_lds(crl::k_shared_persist<8, 2, false, true>, act - kStaticLdsReserve));
+  HIP_TRY(allow_lds(crl::k_shared_persist<4, 1, true, false>, act - kStaticLdsReserve));
+  HIP_TRY(allow_lds(crl::k_shared_persist<4, 1, true, true>, act - kStaticLdsReserve));
+  HIP_TRY(allow_lds(crl::k_shared_persist<4, 2, true, false>, act - kStaticLdsReserve));
+  HIP_TRY(allow_lds(crl::k_shared_persist<4, 2, true, true>, act - kStaticLdsReserve));
+  HIP_TRY(allow_lds(crl::k_shared_persist<8, 1, true, false>, act - kStaticLdsReserve));
+  HIP_TRY(allow_lds(crl::k_shared_persist<8, 1, true, true>, act - kStaticLdsReserve));
+  HIP_TRY(allow_lds(crl::k_shared_persist<8, 2, true, false>, act - kStaticLdsReserve));
+  HIP_TRY(allow_lds(crl::k_shared_persist<8, 2, true, true>, act - kStaticLdsReserve));
   e->lds_opt_in = true;
   return CRL_OK;
 }
@@ -654,6 +662,7 @@ struct PersistPlan {
   bool ok;
   int grid;
   bool lds_map;
+  bool fold;  // the instantiation with the common configuration's rules folded in
   size_t lds;
   crl::ReduceGeom G;
   // what the workgroups exchange, in 64-bit words from the start of one buffer
@@ -680,6 +689,9 @@ PersistPlan plan_persist(const crl_engine* e, int n_steps) {
   p.G.main_shift = crl::main_shift_for(p.G.own_shift);
   p.grid = crl::kPersistMaxGroups;
   p.G.n_blocks = p.grid;  // workgroups without envs hand over empty cells
+  const crl_config& c = e->cfg;
+  p.fold = c.goal_mode == CRL_GOAL_ON_TARGET && c.auto_reset == 1 && c.max_mode == CRL_MAX_TRUE && c.reward_flags == 0 &&
+           e->trace_n == 0 && e->sup_n == 0 && c.max_episodes == 0 && c.track_returns == 0;
   const int n_own = 1 << p.G.own_shift;
   const size_t map_bytes = (size_t)e->map_words * 4;
   p.lds_map = e->cfg.map_mode == CRL_MAP_SHARED && sizeof(crl::PersistLds) + map_bytes <= kLdsPerWorkgroup - kStaticLdsReserve;
@@ -694,7 +706,7 @@ PersistPlan plan_persist(const crl_engine* e, int n_steps) {
   return p;
 }
 
-template <int A, int MAP, bool CLK>
+template <int A, int MAP, bool CLK, bool FOLD>
 hipError_t launch_persist_kernel(crl_engine* e, const PersistPlan& p, unsigned long long* buf, uint64_t t0,
                                  int n_steps, int trace_row0) {
   crl::Rules R = e->rules();
@@ -710,7 +722,7 @@ hipError_t launch_persist_kernel(crl_engine* e, const PersistPlan& p, unsigned l
   void* args[] = {&R, &P, &t0, &n_steps, &trace_row0, &G, &B, &spin_limit};
   // a cooperative launch is refused unless all workgroups can be resident together,
   // which the kernel's waits rely on
-  return hipLaunchCooperativeKernel(reinterpret_cast<const void*>(&crl::k_shared_persist<A, MAP, CLK>), dim3(p.grid),
+  return hipLaunchCooperativeKernel(reinterpret_cast<const void*>(&crl::k_shared_persist<A, MAP, CLK, FOLD>), dim3(p.grid),
                                     dim3(256), args, (unsigned)p.lds, e->stream);
 }
 
@@ -745,8 +757,10 @@ int run_persist(crl_engine* e, int n_steps, bool* launched) {
     const int row0 = (int)std::min<long long>((long long)e->trace_cursor + done, e->trace_cap);
     hipError_t h;
 #define CRL_PERSIST(A, MAP) \
-  (e->persist_clocks ? launch_persist_kernel<A, MAP, true>(e, p, buf, t0, n, row0) \
-                     : launch_persist_kernel<A, MAP, false>(e, p, buf, t0, n, row0))
+  (e->persist_clocks ? (p.fold ? launch_persist_kernel<A, MAP, true, true>(e, p, buf, t0, n, row0)    \
+                               : launch_persist_kernel<A, MAP, true, false>(e, p, buf, t0, n, row0))  \
+                     : (p.fold ? launch_persist_kernel<A, MAP, false, true>(e, p, buf, t0, n, row0)   \
+                               : launch_persist_kernel<A, MAP, false, false>(e, p, buf, t0, n, row0)))
     if (e->A == 4) h = p.lds_map ? CRL_PERSIST(4, 1) : CRL_PERSIST(4, 2);
     else h = p.lds_map ? CRL_PERSIST(8, 1) : CRL_PERSIST(8, 2);
 #undef CRL_PERSIST
@@ -1506,7 +1520,7 @@ int crl_fused_kernel_info(crl_engine* e, int32_t n_steps, char* name, size_t nam
   } else {
     const PersistPlan pp = plan_persist(e, n_steps > 0 ? n_steps : 1 << 20);
     if (pp.ok) {
-      if (name && name_len) snprintf(name, name_len, "k_shared_persist<%d,%d>", e->A, pp.lds_map ? 1 : 2);
+      if (name && name_len) snprintf(name, name_len, "k_shared_persist<%d,%d%s>", e->A, pp.lds_map ? 1 : 2, pp.fold ? ",folded" : "");
       if (grid) *grid = pp.grid;
       if (block) *block = 256;
       if (lds_bytes) *lds_bytes = (int32_t)pp.lds;

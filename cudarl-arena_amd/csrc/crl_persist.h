@@ -128,7 +128,12 @@ __device__ __forceinline__ Row<8> row_of_tagged<8>(const unsigned long long (&v)
 // G.own_shift = kPersistOwnShift, G.n_blocks = 256 = the number of workgroups (blocks
 // without envs hand over empty cells).
 // Everything in B holds tag 0 at launch (cleared by the host), *B.err is zero.
-template <int A, int MAP, bool CLK>
+// FOLD = the rules of the common configuration are compile-time facts (goal test on the
+// target cell, restart at the end of an episode, true maximum, rewards by class, no trace,
+// no supplied stream, no episode budget, no return statistics): the general kernel keeps
+// a dozen lane masks and pointers for them that do not fit the scalar registers and are
+// fetched back again and again (190 lane reads per step).
+template <int A, int MAP, bool CLK, bool FOLD>
 __global__ __launch_bounds__(256) void k_shared_persist(const Rules R, const Ptrs P, const uint64_t t0,
                                                          const int n_steps, const int trace_row0,
                                                          const ReduceGeom G, const PersistBufs B,
@@ -167,14 +172,14 @@ __global__ __launch_bounds__(256) void k_shared_persist(const Rules R, const Ptr
   float reward = has_env ? P.reward[env] : 0.0f;
   int action = has_env ? P.action[env] : 0;
   const int start = has_env ? P.start[env] : 0;
-  const bool track = P.ret_acc != nullptr;
+  const bool track = !FOLD && P.ret_acc != nullptr;
   float ret = (track && has_env) ? P.ret_acc[env] : 0.0f;
   const uint32_t* gmap = P.map + ((P.map_shared || !has_env) ? 0 : (size_t)env * P.map_words);
   const float* cr = P.cell_reward ? P.cell_reward + ((P.map_shared || !has_env) ? 0 : (size_t)env * P.S) : nullptr;
   const DevWindow w_table = dev_window(B.table), w_cells = dev_window(B.cells);
   // 64-bit words of one buffer of main halves; cells with an extension: as many again, behind both buffers
   const size_t cells_half = ((size_t)n_own * G.n_blocks) << G.main_shift;
-  const bool cells_flag = (R.reward_flags & 1) != 0;
+  const bool cells_flag = !FOLD && (R.reward_flags & 1) != 0;
   const bool base_cells = cells_flag && (R.reward_flags & 2) != 0;
 
   // owner: lane l of wave 0 keeps the table value of its key in a register; the A lanes
@@ -229,8 +234,8 @@ __global__ __launch_bounds__(256) void k_shared_persist(const Rules R, const Ptr
   float eps = 0.0f;
   auto prepare = [&](int k) {
     const uint64_t t = t0 + (uint64_t)k;
-    live = has_env && !(R.max_episodes > 0 && episode >= R.max_episodes);
-    if (has_env && !live) trace_idle(P, env, trace_row0 + k, s);
+    live = has_env && (FOLD || !(R.max_episodes > 0 && episode >= R.max_episodes));
+    if (!FOLD && has_env && !live) trace_idle(P, env, trace_row0 + k, s);
     s0 = s;
     const int x0 = s0 % R.W, y0 = s0 / R.W;
     if (live) {
@@ -245,7 +250,7 @@ __global__ __launch_bounds__(256) void k_shared_persist(const Rules R, const Ptr
       mv = moves_of_cell<A>(word_of, R.W, R.H, x0, y0, s0);
       cls0 = cell_class_of(word_of(s0 >> 4), s0);
       d = pick_draw(explore_block(R.seed, (uint32_t)env, t >> 1), t, A);
-      if (P.u_sup && t >= P.sup_t0 && t - P.sup_t0 < (uint64_t)P.sup_n) {
+      if (!FOLD && P.u_sup && t >= P.sup_t0 && t - P.sup_t0 < (uint64_t)P.sup_n) {
         const size_t o = (size_t)(t - P.sup_t0) * P.N + env;
         d.u = P.u_sup[o];
         d.a = P.a_sup[o];
@@ -333,19 +338,19 @@ __global__ __launch_bounds__(256) void k_shared_persist(const Rules R, const Ptr
       const bool moved = code < kTrap;
       const bool trap = code == kTrap;
       const int s2 = moved ? tgt : s0;
-      const bool hit = R.goal_mode == 0 ? code == kGoal : ((moved ? code : cls0) == kGoal);
+      const bool hit = (FOLD || R.goal_mode == 0) ? code == kGoal : ((moved ? code : cls0) == kGoal);
       const float by_class = hit ? R.goal_reward : trap ? R.trap_reward : R.step_reward;
       float by_cell = 0.0f;
       if (cells_flag) by_cell = cr[(trap && !hit) ? tgt : s2];
       reward = (cells_flag && (hit || trap || base_cells)) ? by_cell : by_class;
-      done = hit || (!R.auto_reset && done);
+      done = hit || (!FOLD && !R.auto_reset && done);
       float m = (s2 != s0) ? m_tgt : row_max(row, false, 0);
-      if (R.max_mode == 1) m = fmaxf(0.0f, m);
+      if (!FOLD && R.max_mode == 1) m = fmaxf(0.0f, m);
       m = done ? 0.0f : m;
       my_key = s0 * A + a;
       my_delta = td_delta(row_get(row, a), reward, m, R.lr, R.gamma);
       action = a;
-      if (env < P.trace_n && trace_row0 + k < P.trace_cap) {
+      if (!FOLD && env < P.trace_n && trace_row0 + k < P.trace_cap) {
         const size_t o = (size_t)(trace_row0 + k) * P.trace_n + env;
         P.tr_s[o] = s2;
         P.tr_a[o] = (uint8_t)a;
@@ -354,7 +359,7 @@ __global__ __launch_bounds__(256) void k_shared_persist(const Rules R, const Ptr
       }
       ep_step += 1;
       ret = ret + reward;
-      if (R.auto_reset && (done || (R.episode_len > 0 && ep_step >= R.episode_len))) {
+      if ((FOLD || R.auto_reset) && (done || (R.episode_len > 0 && ep_step >= R.episode_len))) {
         if (track) record_episode(P, env, ret, ep_step);
         ret = 0.0f;
         s = start;

@@ -387,11 +387,11 @@ def test_shared_table_one_launch_kernel_shapes(gpu, oracle):
     cfg = gpu.make_config(300, 16, 16, table_mode=gpu.TABLE_SHARED, map_mode=gpu.MAP_SHARED, lr=0.01, eps0=0.3,
                           episode_len=25, seed=3, trap_reward=-0.5)
     with gpu.Engine(cfg, 0) as eng:
-        assert eng.fused_kernel_info(10)["name"] == "k_shared_persist<4,1>"  # (automatic)
+        assert eng.fused_kernel_info(10)["name"] == "k_shared_persist<4,1,folded>"  # (automatic; the common rules)
         eng.set_fused_variant(1)
         assert eng.fused_kernel_info(10)["name"] == "k_shared_act+k_reduce_owners"
         eng.set_fused_variant(2)
-        assert eng.fused_kernel_info(1)["name"] == "k_shared_persist<4,1>" and eng.fused_kernel_info(1)["grid"] == 256
+        assert eng.fused_kernel_info(1)["name"] == "k_shared_persist<4,1,folded>" and eng.fused_kernel_info(1)["grid"] == 256
     run_both(gpu, oracle, cfg, cls, start, 90, chunks=[1, 30, 1, 1, 50, 7], variant=2)
     # 8 actions, cell rewards, per-env maps (global memory), linear epsilon, 1000 envs: last block 232 envs
     N, W, H = 1000, 24, 20
@@ -494,7 +494,7 @@ def test_shared_table_automatic_plan_and_cell_sizes(gpu, oracle):
                               episode_len=30, seed=4, trap_reward=-0.5)
         with gpu.Engine(cfg, 0) as eng:
             name = eng.fused_kernel_info(50)["name"]
-            assert name == ("k_shared_persist<4,1>" if auto == "persist" else "k_shared_act+k_reduce_owners"), (W, H, name)
+            assert name == ("k_shared_persist<4,1,folded>" if auto == "persist" else "k_shared_act+k_reduce_owners"), (W, H, name)
             assert eng.fused_kernel_info(1)["name"] == "k_shared_act+k_reduce_owners"  # too short to repay the set-up
         for variant in (1, 2):
             _, q = run_both(gpu, oracle, cfg, cls, start, 40, variant=variant)
