@@ -325,6 +325,9 @@ __global__ __launch_bounds__(256) void k_shared_persist(const Rules R, const Ptr
     if (live) {
       const Row<A> row = row_of_tagged<A>(rq);
       const int a = (d.u < eps) ? d.a : row_argmax(row);
+      // (the key is known: its leader is being found while the delta is worked out)
+      my_key = s0 * A + a;
+      atomicMin(&L.red.lead[my_key], (uint32_t)tid);
       // the rule of step_rule() on the move code of the action: the class of the target
       // cell, or kWall outside the grid
       const int code = (int)((mv >> (2 * a)) & 3u);
@@ -376,7 +379,7 @@ __global__ __launch_bounds__(256) void k_shared_persist(const Rules R, const Ptr
     // (`sorted`: the upper half of the tile, which is free until the block sums are through)
     const bool over = reduce_block<true>(L.red, G, wg, my_key, my_delta, live, B.cells, want, L.tile + kTileBlocks * kOwnKeys / 2,
                                          L.stage, &w_cells,
-                                         (uint32_t)((size_t)half * cells_half * 8), B.cells + (2 + half) * cells_half);
+                                         (uint32_t)((size_t)half * cells_half * 8), B.cells + (2 + half) * cells_half, true);
     if (over && has_env)
       st_dev64(B.raw + (size_t)half * P.N + env, tagged(__float_as_uint(my_delta),
                                    (uint32_t)my_key | (live ? kRawValid : 0u) | (want << kRawTagShift)));
@@ -453,10 +456,13 @@ __global__ __launch_bounds__(256) void k_shared_persist(const Rules R, const Ptr
             if (cnt[j] == kSlotOverflow) {
               if (pair == 0) L.o_list[atomicAdd(&L.o_count, 1)] = (uint8_t)blk;
             } else {
-              if (2 * pair < cnt[j]) row[rec_slot(rec[j].x)] = __uint_as_float(rec[j].y);
-              if (2 * pair + 1 < cnt[j]) row[rec_slot(rec[j].z)] = __uint_as_float(rec[j].w);
-              if (kMainRecs + 2 * pair < cnt[j]) row[rec_slot(more[j].x)] = __uint_as_float(more[j].y);
-              if (kMainRecs + 2 * pair + 1 < cnt[j]) row[rec_slot(more[j].z)] = __uint_as_float(more[j].w);
+              // (no branches: a record that is not there goes to a word of this thread's that
+              // nobody reads)
+              float* none = &L.o_delta[tid];
+              *(2 * pair < cnt[j] ? &row[rec_slot(rec[j].x)] : none) = __uint_as_float(rec[j].y);
+              *(2 * pair + 1 < cnt[j] ? &row[rec_slot(rec[j].z)] : none) = __uint_as_float(rec[j].w);
+              *(kMainRecs + 2 * pair < cnt[j] ? &row[rec_slot(more[j].x)] : none) = __uint_as_float(more[j].y);
+              *(kMainRecs + 2 * pair + 1 < cnt[j] ? &row[rec_slot(more[j].z)] : none) = __uint_as_float(more[j].w);
             }
           }
         }

@@ -205,12 +205,13 @@ __device__ __forceinline__ bool reduce_block(ReduceLds& L, const ReduceGeom G, c
                                              const int key, const float delta, const bool valid,
                                              unsigned long long* handoff, const uint32_t tag, float* sorted,
                                              unsigned long long* stage = nullptr, const DevWindow* window = nullptr,
-                                             const uint32_t window_offset = 0, unsigned long long* ext = nullptr) {
+                                             const uint32_t window_offset = 0, unsigned long long* ext = nullptr,
+                                             const bool elected = false) {
   const int tid = threadIdx.x;
   const int n_own = 1 << G.own_shift;
   const int cap = 1 << G.cell_shift;  // records of a cell
   const int cap_main = 1 << G.main_shift;  // DEV: of its main half
-  if (valid) atomicMin(&L.lead[key], (uint32_t)tid);
+  if (valid && !elected) atomicMin(&L.lead[key], (uint32_t)tid);  // (elected: the caller has done this already)
   L.delta[tid] = delta;
   __syncthreads();
   L.handed[tid] = 0;  // (256 >= owners; the last call's readers are past the barrier above)
