@@ -324,7 +324,8 @@ __global__ __launch_bounds__(256) void k_shared_persist(const Rules R, const Ptr
     float my_delta = 0.0f;
     if (live) {
       const Row<A> row = row_of_tagged<A>(rq);
-      const int a = (d.u < eps) ? d.a : row_argmax(row);
+      const int greedy = row_argmax(row);  // (worked out for every env: cheaper than a branch around it)
+      const int a = (d.u < eps) ? d.a : greedy;
       // (the key is known: its leader is being found while the delta is worked out)
       my_key = s0 * A + a;
       atomicMin(&L.red.lead[my_key], (uint32_t)tid);
@@ -362,15 +363,12 @@ __global__ __launch_bounds__(256) void k_shared_persist(const Rules R, const Ptr
       }
       ep_step += 1;
       ret = ret + reward;
-      if ((FOLD || R.auto_reset) && (done || (R.episode_len > 0 && ep_step >= R.episode_len))) {
-        if (track) record_episode(P, env, ret, ep_step);
-        ret = 0.0f;
-        s = start;
-        ep_step = 0;
-        episode += 1;
-      } else {
-        s = s2;
-      }
+      const bool over_now = (FOLD || R.auto_reset) && (done || (R.episode_len > 0 && ep_step >= R.episode_len));
+      if (!FOLD && track && over_now) record_episode(P, env, ret, ep_step);
+      ret = over_now ? 0.0f : ret;
+      s = over_now ? start : s2;
+      ep_step = over_now ? 0 : ep_step;
+      episode += over_now ? 1 : 0;
     }
     CRL_MARK(2);
 
@@ -453,17 +451,18 @@ __global__ __launch_bounds__(256) void k_shared_persist(const Rules R, const Ptr
           for (int j = 0; j < GS; ++j) {
             const int blk = wave * 64 + j * 32 + (lane >> 1);
             float* row = L.tile + blk * kOwnKeys;
-            if (cnt[j] == kSlotOverflow) {
-              if (pair == 0) L.o_list[atomicAdd(&L.o_count, 1)] = (uint8_t)blk;
-            } else {
-              // (no branches: a record that is not there goes to a word of this thread's that
-              // nobody reads)
-              float* none = &L.o_delta[tid];
-              *(2 * pair < cnt[j] ? &row[rec_slot(rec[j].x)] : none) = __uint_as_float(rec[j].y);
-              *(2 * pair + 1 < cnt[j] ? &row[rec_slot(rec[j].z)] : none) = __uint_as_float(rec[j].w);
-              *(kMainRecs + 2 * pair < cnt[j] ? &row[rec_slot(more[j].x)] : none) = __uint_as_float(more[j].y);
-              *(kMainRecs + 2 * pair + 1 < cnt[j] ? &row[rec_slot(more[j].z)] : none) = __uint_as_float(more[j].w);
+            const bool too_many = cnt[j] == kSlotOverflow;
+            if (__any(too_many)) {  // (rare)
+              if (too_many && pair == 0) L.o_list[atomicAdd(&L.o_count, 1)] = (uint8_t)blk;
             }
+            // (no branches: a record that is not there goes to a word of this thread's that
+            // nobody reads)
+            const int n = too_many ? 0 : cnt[j];
+            float* none = &L.o_delta[tid];
+            *(2 * pair < n ? &row[rec_slot(rec[j].x)] : none) = __uint_as_float(rec[j].y);
+            *(2 * pair + 1 < n ? &row[rec_slot(rec[j].z)] : none) = __uint_as_float(rec[j].w);
+            *(kMainRecs + 2 * pair < n ? &row[rec_slot(more[j].x)] : none) = __uint_as_float(more[j].y);
+            *(kMainRecs + 2 * pair + 1 < n ? &row[rec_slot(more[j].z)] : none) = __uint_as_float(more[j].w);
           }
         }
       }
