@@ -228,10 +228,13 @@ __device__ __forceinline__ bool reduce_block(ReduceLds& L, const ReduceGeom G, c
   // leader's walk is loads from known addresses, several in flight, instead of one bit
   // scan, load and add after the other (envs that crowd on a few cells: 14 holders of
   // one key in most blocks, 1 us of such a walk).
+  // (Written without branches: one wave to a SIMD has nothing to hide them behind.  A thread
+  // without a sample reads its own, empty member set; a thread that has nothing to line up
+  // writes its delta where it already is.)
   const bool leader = valid && ld == (uint32_t)tid;
-  unsigned long long mw[4] = {0ull, 0ull, 0ull, 0ull};
-  int holders = 0;  // leader: the key's further holders
-  if (valid) {
+  unsigned long long mw[4];
+  int holders;  // leader: the key's further holders
+  {
     const ulonglong2 lo = *reinterpret_cast<const ulonglong2*>(&L.members[ld][0]);
     const ulonglong2 hi = *reinterpret_cast<const ulonglong2*>(&L.members[ld][2]);
     mw[0] = lo.x;
@@ -239,14 +242,12 @@ __device__ __forceinline__ bool reduce_block(ReduceLds& L, const ReduceGeom G, c
     mw[2] = hi.x;
     mw[3] = hi.y;
     const int p0 = __popcll(mw[0]), p1 = __popcll(mw[1]), p2 = __popcll(mw[2]), p3 = __popcll(mw[3]);
-    if (leader) {
-      holders = p0 + p1 + p2 + p3;
-    } else {
-      const int w = tid >> 6;
-      const unsigned long long mine = w == 0 ? mw[0] : w == 1 ? mw[1] : w == 2 ? mw[2] : mw[3];
-      const int place = (w > 0 ? p0 : 0) + (w > 1 ? p1 : 0) + (w > 2 ? p2 : 0) + __popcll(mine & ((1ull << (tid & 63)) - 1ull));
-      if (place < kSortRows) sorted[place * kBlockSamples + (int)ld] = delta;
-    }
+    holders = leader ? p0 + p1 + p2 + p3 : 0;
+    const int w = tid >> 6;
+    const unsigned long long mine = w == 0 ? mw[0] : w == 1 ? mw[1] : w == 2 ? mw[2] : mw[3];
+    const int place = (w > 0 ? p0 : 0) + (w > 1 ? p1 : 0) + (w > 2 ? p2 : 0) + __popcll(mine & ((1ull << (tid & 63)) - 1ull));
+    const bool lines_up = valid && !leader && place < kSortRows;
+    *(lines_up ? &sorted[place * kBlockSamples + (int)ld] : &L.delta[tid]) = delta;
   }
   __syncthreads();
   float acc = 0.0f;
