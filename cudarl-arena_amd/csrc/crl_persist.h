@@ -58,8 +58,6 @@ static_assert(main_shift_for(kPersistOwnShift) == kMainShift && cell_shift_for(k
               (1 << kPersistOwnShift) == kPersistMaxGroups && (kPersistMaxGroups << (kMainShift - 1)) == kStagePieces,
               "the owner's loads are laid out for cells of 4 + 4 records");
 constexpr int kPersistMaxSteps = 65535;     // per launch: the raw samples' tags have 17 bits
-constexpr int kPersistTablePause = 1;       // x 128 clocks between a step's preparation and its first look at the table
-constexpr int kPersistCellsPause = 1;       // x 128 clocks between clearing the tile and the first look at the cells
 constexpr int kPersistClockWords = 20 + 8 * 256;  // 2 workgroups x (8 phases + polls of the two waits by thread 0),
                                                   // then the wall clock of every workgroup at the 8 marks of one step
 
@@ -271,11 +269,10 @@ __global__ __launch_bounds__(256) void k_shared_persist(const Rules R, const Ptr
     // (the values this workgroup published as an owner are on their way meanwhile)
     prepare(k);
     reduce_stage_init(L.stage, G, want);
-    // A first look that comes too early costs a whole round trip more than one that comes
-    // just in time: the values published at the end of the last step need about 1.5 us to
-    // be visible, the preparation above takes 1 us (65,536 envs on 64x64x4, us per step by
-    // pause: none 7.10, 2 x 128 clocks 6.98, 4 x 7.04, 6 x 7.14, 8 x 7.24).
-    for (int i = 0; i < kPersistTablePause; ++i) __builtin_amdgcn_s_sleep(2);
+    // (The values published at the end of the last step need about 1 us to be visible, which
+    // is what the preparation above takes.  A look that comes too early costs a whole round
+    // trip more; while a step was longer than now, a pause of 0.1-0.2 us here and before the
+    // first look at the cells was worth 0.1-0.4 us per step, and now it no longer is.)
     CRL_MARK(0);
 
 
@@ -389,10 +386,8 @@ __global__ __launch_bounds__(256) void k_shared_persist(const Rules R, const Ptr
 #pragma unroll
       for (int i = 0; i < kTileBlocks * kOwnKeys / 4 / 256; ++i) tile4[i * 64 + lane] = make_float4(0.0f, 0.0f, 0.0f, 0.0f);
     }
-    // A short pause before the first look at the others' cells: asking while the own
-    // stores have only just left takes longer (no pause 7.06 us per step, 4 x 128 clocks
-    // 6.97, 8 x 7.03, 12 x 7.56; waiting until the 8 KB of own cells are acknowledged 7.30).
-    for (int i = 0; i < kPersistCellsPause; ++i) __builtin_amdgcn_s_sleep(2);
+    // (no waiting for the own cells' acknowledgement before the first look at the others':
+    // that costs 0.3 us per step; clearing the tile first is pause enough)
     if (L.dead) {  // some thread gave up waiting for the table
       gave_up = true;
       break;
