@@ -522,7 +522,8 @@ bool reduce_fast(const crl_engine* e, const crl::ReduceGeom& G) {
 }
 
 constexpr size_t kOwnersLds = (size_t)(crl::kTileBlocks + crl::kTileBlocks / crl::kGroupBlocks) *
-                              crl::kOwnKeys * sizeof(float);
+                              crl::kOwnKeys * sizeof(float) +
+                              crl::kBlockSamples * sizeof(float);  // tile, group sums, a word per thread that nobody reads
 
 template <class Kern>
 hipError_t allow_lds(Kern kern, size_t bytes) {

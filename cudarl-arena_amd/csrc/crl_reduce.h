@@ -354,7 +354,7 @@ __global__ __launch_bounds__(256) void k_reduce_owners(const ReduceGeom G, float
                                                         const int32_t* __restrict__ key,
                                                         const float* __restrict__ delta, const int n,
                                                         const unsigned long long* __restrict__ handoff) {
-  extern __shared__ __align__(16) float tile[];  // [kTileBlocks][64] block sums, then [16][64] group sums
+  extern __shared__ __align__(16) float tile[];  // [kTileBlocks][64] block sums, then [16][64] group sums, then a word per thread
   float* gsum = tile + kTileBlocks * kOwnKeys;
   const int tid = threadIdx.x;
   const int lane = tid & 63;
@@ -387,10 +387,12 @@ __global__ __launch_bounds__(256) void k_reduce_owners(const ReduceGeom G, float
     const int c = rec_count(cell[0].x);
     if (c != kSlotOverflow) {
       float* row = tile + tid * kOwnKeys;
+      // (no branches: a record that is not there goes to a word that nobody reads)
+      float* none = gsum + 16 * kOwnKeys + tid;
 #pragma unroll
       for (int i = 0; i < kMinCellRecs / 2; ++i) {
-        if (c > 2 * i) row[rec_slot(cell[i].x)] = __uint_as_float(cell[i].y);
-        if (c > 2 * i + 1) row[rec_slot(cell[i].z)] = __uint_as_float(cell[i].w);
+        *(c > 2 * i ? &row[rec_slot(cell[i].x)] : none) = __uint_as_float(cell[i].y);
+        *(c > 2 * i + 1 ? &row[rec_slot(cell[i].z)] : none) = __uint_as_float(cell[i].w);
       }
       for (int i = kMinCellRecs / 2; 2 * i < c; ++i) {
         const uint4 more = src[i];
@@ -409,14 +411,23 @@ __global__ __launch_bounds__(256) void k_reduce_owners(const ReduceGeom G, float
       }
     }
     __syncthreads();
-    // group sums: 16 groups of 16 blocks in this tile, four per wave; lane = key slot
+    // group sums: 16 groups of 16 blocks in this tile, four per wave; a lane takes four
+    // keys of one group (16 LDS loads of 16 bytes instead of 64 of 4)
+    {
+      const int grp = wave * 4 + (lane >> 4);
+      const float4* rows = reinterpret_cast<const float4*>(tile + grp * kGroupBlocks * kOwnKeys) + (lane & 15);
+      float4 v[kGroupBlocks];
 #pragma unroll
-    for (int gi = 0; gi < 4; ++gi) {
-      const int grp = wave * 4 + gi;
-      float acc = 0.0f;
+      for (int bb = 0; bb < kGroupBlocks; ++bb) v[bb] = rows[bb * (kOwnKeys / 4)];
+      float4 acc = make_float4(0.0f, 0.0f, 0.0f, 0.0f);
 #pragma unroll
-      for (int bb = 0; bb < kGroupBlocks; ++bb) acc = acc + tile[(grp * kGroupBlocks + bb) * kOwnKeys + lane];
-      gsum[grp * kOwnKeys + lane] = acc;
+      for (int bb = 0; bb < kGroupBlocks; ++bb) {
+        acc.x = acc.x + v[bb].x;
+        acc.y = acc.y + v[bb].y;
+        acc.z = acc.z + v[bb].z;
+        acc.w = acc.w + v[bb].w;
+      }
+      reinterpret_cast<float4*>(gsum + grp * kOwnKeys)[lane & 15] = acc;
     }
     __syncthreads();
     if (wave == 0) {
