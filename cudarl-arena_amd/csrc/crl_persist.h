@@ -110,7 +110,8 @@ __device__ __forceinline__ Row<8> row_of_tagged<8>(const unsigned long long (&v)
 // Phase clocks (CLK only): thread 0 of the first and the last workgroup add up the shader
 // clocks between the marks of a step.  Phases: 0 work before the table is needed, 1 wait
 // for the table, 2 select / move / delta, 3 ordered block sums + cells, 4 clearing the
-// tile, 5 wait for the cells, 6 tile + sums + publish, 7 loop overhead.
+// tile, 5 wait for the cells and put them into the tile, 6 group sums + barrier + totals +
+// publish, 7 loop overhead.
 #define CRL_MARK(i)                                                                         \
   do {                                                                                      \
     if (CLK) {                                                                              \
@@ -348,7 +349,6 @@ __global__ __launch_bounds__(256) void k_shared_persist(const Rules R, const Ptr
       float m = (s2 != s0) ? m_tgt : row_max(row, false, 0);
       if (!FOLD && R.max_mode == 1) m = fmaxf(0.0f, m);
       m = done ? 0.0f : m;
-      my_key = s0 * A + a;
       my_delta = td_delta(row_get(row, a), reward, m, R.lr, R.gamma);
       action = a;
       if (!FOLD && env < P.trace_n && trace_row0 + k < P.trace_cap) {
