@@ -41,7 +41,7 @@ WORKLOADS = {
     # launch_steps: env-steps every env takes in one pass (the configuration's own length)
     "c2": dict(n=4096, launch_steps=10000, bytes=42.5, traffic=8.2,
                name="c2: 4096 envs 32x32, per-env tables 1024x4, eps 0.1, T=256, 10000 steps"),
-    "c3": dict(n=65536, launch_steps=1000, bytes=24.0,
+    "c3": dict(n=65536, launch_steps=1000, bytes=24.0, traffic=173.9,
                name="c3: 65536 envs, shared 64x64 map, one shared table 4096x4, ordered reduction, "
                     "lr 0.05 (as specified: the table overflows within ~100 steps), 1000 steps"),
     # the same with a step size small enough for the table to stay finite, so that the
