@@ -30,8 +30,10 @@
 //   block:  what does not depend on the table (exploration draw, neighbour cells, move
 //           codes; the owner's stores are on their way meanwhile) -> poll the view of
 //           the env's cell -> select, move, (key, delta) -> ordered block sums -> cells
-//   owner:  clear the tile, a short pause -> poll the cells of all blocks -> tile ->
-//           sums in tree order -> new values and row maxima into the views
+//   owner:  wave by wave (64 blocks = four groups of the tree each): clear the wave's
+//           quarter of the tile -> poll the cells of its blocks -> into the tile -> its
+//           four group sums; one barrier; totals in group order -> new values and row
+//           maxima into the views
 // An owner overwrites its values only after it has every block's cells of the step,
 // which a block writes after all its threads have read theirs: one buffer of views
 // suffices.  Cells and raw samples have two buffers, taken in turn: a workgroup that
