@@ -184,7 +184,8 @@ __global__ __launch_bounds__(256) void k_shared_persist(const Rules R, const Ptr
   const bool base_cells = cells_flag && (R.reward_flags & 2) != 0;
 
   // owner: lane l of wave 0 keeps the table value of its key in a register; the A lanes
-  // of a row sit side by side, the first of them also publishes the row's maximum
+  // of a row sit side by side, each of them publishes its value and one copy of the row's
+  // maximum
   const int own_key = key_of(wg, lane, G);
   const bool own_live = wave == 0 && own_key < G.K;
   float q_own = own_live ? P.Q[own_key] : 0.0f;
@@ -225,8 +226,8 @@ __global__ __launch_bounds__(256) void k_shared_persist(const Rules R, const Ptr
   if (wave == 0) publish(1u);
   __syncthreads();
 
-  // What a step needs that does not depend on the table: computed for step k + 1 while
-  // the cells of step k are on their way to the owners.
+  // What a step needs that does not depend on the table: computed at the top of the step,
+  // while the values of the step before are on their way from the owners.
   bool live = false;
   int s0 = 0, cls0 = kFree;
   int nb[A];
@@ -277,7 +278,6 @@ __global__ __launch_bounds__(256) void k_shared_persist(const Rules R, const Ptr
     // trip more; while a step was longer than now, a pause of 0.1-0.2 us here and before the
     // first look at the cells was worth 0.1-0.4 us per step, and now it no longer is.)
     CRL_MARK(0);
-
 
     // ---- the table of this step: the view of the env's cell ----------------------------
     unsigned long long rq[A], rn[A];
@@ -382,7 +382,7 @@ __global__ __launch_bounds__(256) void k_shared_persist(const Rules R, const Ptr
                                    (uint32_t)my_key | (live ? kRawValid : 0u) | (want << kRawTagShift)));
     CRL_MARK(3);
 
-    // ---- while the cells travel: the owner's tile cleared, the next step prepared ----
+    // ---- while the cells travel: the owner's tile cleared -------------------------------
     {  // (each wave its own quarter)
       float4* tile4 = reinterpret_cast<float4*>(L.tile) + wave * (kTileBlocks * kOwnKeys / 4 / 4);
 #pragma unroll
